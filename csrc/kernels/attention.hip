@@ -55,6 +55,11 @@ struct Scaler {
   // head of its kv group sees (bs_stage_needed) before loading them.
   int bs_shift, bs_local, bs_vert, bs_step, bs_h0;
   int bs_skip;   // prefill skips invisible stages (OME_BS_SKIP=0: mask only, the r05 behaviour)
+  // Kept first tokens of a sliding window: keys [0, keep) stay visible (at their true positions)
+  // after they left the window, i.e. key j is seen by query i when j <= i and (i - j < window or
+  // j < keep).  0 = off.  Kernels skip the key tiles that lie wholly between the two ranges.
+  int keep;
+  __device__ __forceinline__ bool in_window(int key, int lo) const { return key >= lo || key < keep; }
   __device__ __forceinline__ float alibi_l2(int head) const {
     return alibi != nullptr ? alibi[head] * 1.4426950408889634f : 0.f;
   }
@@ -117,6 +122,7 @@ static inline Scaler make_scaler(float scale, float softcap, const float* alibi 
   Scaler r;
   r.alibi = alibi;
   r.row_lo = nullptr;
+  r.keep = 0;
   set_blocksparse(r, bs);
   r.mul = scale * l2e;
   r.cap_inv = softcap > 0.f ? scale / softcap : 0.f;
@@ -385,8 +391,8 @@ __device__ __forceinline__ void kv_tile_compute(const KVTile<D, F>& t, const bf1
   for (int i = 0; i < 4; ++i) {
     const int k0 = kb + 4 * g + i, k1 = k0 + 16;
     // AL instantiation: ALiBi bias and / or the block-sparse mask (both per query head)
-    const bool v0 = k0 < p_end && k0 >= lo && (!AL || scl.bs_visible(qpos, k0, head));
-    const bool v1 = k1 < p_end && k1 >= lo && (!AL || scl.bs_visible(qpos, k1, head));
+    const bool v0 = k0 < p_end && (AL ? scl.in_window(k0, lo) : k0 >= lo) && (!AL || scl.bs_visible(qpos, k0, head));
+    const bool v1 = k1 < p_end && (AL ? scl.in_window(k1, lo) : k1 >= lo) && (!AL || scl.bs_visible(qpos, k1, head));
     s0[i] = v0 ? (AL ? scl(s0[i]) + al * (float)(k0 - qpos) : scl(s0[i])) : OME_NEG_INF;
     s1[i] = v1 ? (AL ? scl(s1[i]) + al * (float)(k1 - qpos) : scl(s1[i])) : OME_NEG_INF;
     mt = fmaxf(mt, fmaxf(s0[i], s1[i]));
@@ -460,8 +466,8 @@ __device__ __forceinline__ void kv_tilep_compute(const KVTileP<D, F>& t, const b
   for (int i = 0; i < 4; ++i) {
     const int k0 = base + i, k1 = k0 + 4;
     // AL instantiation: ALiBi bias and / or the block-sparse mask (both per query head)
-    const bool v0 = k0 < p_end && k0 >= lo && (!AL || scl.bs_visible(qpos, k0, head));
-    const bool v1 = k1 < p_end && k1 >= lo && (!AL || scl.bs_visible(qpos, k1, head));
+    const bool v0 = k0 < p_end && (AL ? scl.in_window(k0, lo) : k0 >= lo) && (!AL || scl.bs_visible(qpos, k0, head));
+    const bool v1 = k1 < p_end && (AL ? scl.in_window(k1, lo) : k1 >= lo) && (!AL || scl.bs_visible(qpos, k1, head));
     s0[i] = v0 ? (AL ? scl(s0[i]) + al * (float)(k0 - qpos) : scl(s0[i])) : OME_NEG_INF;
     s1[i] = v1 ? (AL ? scl(s1[i]) + al * (float)(k1 - qpos) : scl(s1[i])) : OME_NEG_INF;
     mt = fmaxf(mt, fmaxf(s0[i], s1[i]));
@@ -532,14 +538,15 @@ __global__ __launch_bounds__(256) void paged_decode_v2_kernel(
   const int* bt = block_tables + (int64_t)b * bt_stride;
   const int64_t kpage = (int64_t)Hkv * P * D;
   int kb = p_start + wave * 32;
-  if (lo > 0) {  // sliding window: skip whole tiles before the window
-    while (kb + 32 <= lo && kb < p_end) kb += 128;
+  if (lo > 0) {  // sliding window: skip whole tiles before the window (not the kept first keys)
+    while (kb + 32 <= lo && kb >= scl.keep && kb < p_end) kb += 128;
   }
   if (MODE == 2) {
     const int qb = AL && scl.bs_shift ? qpos >> scl.bs_shift : 0;
     for (; kb < p_end; kb += 128) {
       // block-sparse: a 32-key tile no head of the group sees is not loaded at all
       if (AL && scl.bs_shift && scl.bs_skip && !scl.bs_stage_needed(kb, 32, qb, kvh * G, G)) continue;
+      if (AL && kb >= scl.keep && kb + 32 <= lo) continue;   // between the kept keys and the window
       KVTileP<D, F> t;
       kv_tilep_load<D, P, F>(t, k_cache, v_cache, bt, kb, seq_len, kpage, kvh, n, g);
       kv_tilep_compute<D, F, AL>(t, qf, o, m_i, l_i, kb, p_end, lo, scl, g, al, qpos, kvh * G + n);
@@ -618,7 +625,7 @@ static void launch_decode_v2(int variant, dim3 grid, size_t smem, hipStream_t st
                              int window, const int* order, float v_scale, const float* sinks) {
   // ALiBi (Bloom / MPT) runs the key-permuted variant only, compiled with the bias term; the
   // other instantiations carry no trace of it
-  auto kern = (scl.alibi != nullptr || scl.bs_shift != 0) ? paged_decode_v2_kernel<D, 16, 2, F, true>
+  auto kern = (scl.alibi != nullptr || scl.bs_shift != 0 || scl.keep > 0) ? paged_decode_v2_kernel<D, 16, 2, F, true>
               : variant == 2       ? paged_decode_v2_kernel<D, 16, 1, F>
               : variant == 4       ? paged_decode_v2_kernel<D, 16, 2, F>
                                    : paged_decode_v2_kernel<D, 16, 0, F>;
@@ -660,7 +667,7 @@ OME_API int ome_paged_decode(const void* q, int64_t q_stride, const void* k_cach
                              int64_t out_stride, void* part_o, void* part_ml, int B, int Hq, int Hkv, int D, int P,
                              int part_size, int max_parts, float scale, int window, const int* order, int kv_fmt,
                              float k_scale, float v_scale, float softcap, const float* sinks, const float* alibi,
-                             const int* row_lo, int64_t bsparse, hipStream_t stream) {
+                             const int* row_lo, int64_t bsparse, int keep_first, hipStream_t stream) {
   if (B <= 0) return 0;
   if ((D != 64 && D != 128 && D != 256) || P != 16) return -2;
   if (Hq % Hkv != 0 || Hq / Hkv > 16) return -3;
@@ -668,13 +675,14 @@ OME_API int ome_paged_decode(const void* q, int64_t q_stride, const void* k_cach
   if (kv_fmt < 0 || kv_fmt > 2) return -5;
   Scaler scl = make_scaler(scale * k_scale, softcap, alibi, bsparse);
   scl.row_lo = row_lo;
+  scl.keep = window > 0 && keep_first > 0 ? keep_first : 0;
   dim3 grid(max_parts, Hkv, B);
   // A/B switch for benchmarking: 1 = v1, 2 = v2 (register ring), 3 = v2 without ring, 4 = v3 with
   // key-permuted tiles (16-B V loads; default: 5.38 vs 5.24 TB/s on the bench's context mix)
   const char* ve = getenv("OME_DECODE_ATTN");
   int variant = ve ? atoi(ve) : 4;
   if (variant == 1 && (kv_fmt != KV_BF16 || D != 128 || softcap > 0.f || sinks || alibi || row_lo || part_size == 0 ||
-                       scl.bs_shift != 0))
+                       scl.bs_shift != 0 || scl.keep > 0))
     variant = 4;  // v1: plain bf16 D=128, fixed partitions
   if (variant == 1) {
     const size_t smem = (128 + 4 * 16 * D) * sizeof(float);
@@ -730,8 +738,10 @@ __global__ __launch_bounds__(512) void paged_prefill_kernel(
   // row_hi (optional, per query row): last visible key beyond the causal one (Gemma 3 image
   // blocks attend bidirectionally); keys up to the sequence end may then be visible
   const int kv_end = row_hi ? kv_len : min(kv_len, prefix + r_hi);
-  int kv_lo = 0;
-  kv_lo = attn_lo(prefix + r0, window) & ~31;
+  // keys of the item: [kv_lo, kv_end), or with kept first keys [0, keep_end) + [win_lo, kv_end)
+  const int win_lo = attn_lo(prefix + r0, window) & ~31;
+  const int keep_end = (scl.keep + 31) & ~31;
+  const int kv_lo = scl.keep > 0 ? 0 : win_lo;
   const int* bt = block_tables + (int64_t)s * bt_stride;
   const int64_t kpage = (int64_t)Hkv * P * D;
 
@@ -754,6 +764,7 @@ __global__ __launch_bounds__(512) void paged_prefill_kernel(
       for (int nb = 0; nb < NB; ++nb) o[rb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     for (int kb = kv_lo; kb < kv_end; kb += 32) {
+      if (kb >= keep_end && kb < win_lo) kb = win_lo;   // jump from the kept keys to the window
       const int pA = bt[kb / P];
       const int pB = (kb + P < kv_len) ? bt[kb / P + 1] : pA;
       const typename KVStore<F>::T* kA = k_cache + pA * kpage + (int64_t)kvh * P * D;
@@ -788,7 +799,7 @@ __global__ __launch_bounds__(512) void paged_prefill_kernel(
             const int key = kb + 16 * X + 4 * g + i;
             if (al != 0.f) v += al * (float)(key - qpos);
             if (need_mask) {
-              const bool ok = key <= qlim && key < kv_len && key >= attn_lo(qpos, window) &&
+              const bool ok = key <= qlim && key < kv_len && scl.in_window(key, attn_lo(qpos, window)) &&
                                scl.bs_visible(qpos, key, head);
               v = ok ? v : OME_NEG_INF;
             }
@@ -1033,7 +1044,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void paged_prefill_v2_kernel(
               const int key = kbu + 16 * X + 4 * g + i;
               if (al != 0.f) v += al * (float)(key - qpos);
               if (need_mask) {
-                const bool ok = key <= qlim && key < kv_len && key >= attn_lo(qpos, window) &&
+                const bool ok = key <= qlim && key < kv_len && scl.in_window(key, attn_lo(qpos, window)) &&
                                scl.bs_visible(qpos, key, head);
                 v = ok ? v : OME_NEG_INF;
               }
@@ -1399,17 +1410,19 @@ OME_API int ome_paged_prefill(const void* q, int64_t q_stride, const void* k_cac
                               const int* items, int n_items, void* out, int64_t out_stride, int Hq, int Hkv, int D,
                               int P, float scale, int window, int kv_fmt, float k_scale, float v_scale,
                               float softcap, const float* sinks, const float* alibi, const int* row_hi,
-                              int rows, int64_t bsparse, hipStream_t stream) {
+                              int rows, int64_t bsparse, int keep_first, hipStream_t stream) {
   if (n_items <= 0) return 0;
   if (rows != 32 && rows != 64) return -2;
   if ((D != 64 && D != 128 && D != 256) || P != 16) return -2;
   if (Hq % Hkv != 0) return -3;
   if (kv_fmt < 0 || kv_fmt > 2) return -5;
   const int G = Hq / Hkv;
-  const Scaler scl = make_scaler(scale * k_scale, softcap, alibi, bsparse);
+  Scaler scl = make_scaler(scale * k_scale, softcap, alibi, bsparse);
+  scl.keep = window > 0 && keep_first > 0 ? keep_first : 0;
   dim3 grid(n_items, Hkv);
   const char* ve = getenv("OME_PREFILL_ATTN");
-  const int variant = ve ? atoi(ve) : 2;
+  // kept first keys: the classic kernel (it jumps from the kept tiles to the window's)
+  const int variant = scl.keep > 0 ? 0 : ve ? atoi(ve) : 2;
   // 64-row items exist only for the 8-wave GQA-4 / D = 128 kernel; every other kernel would
   // treat them as 32-row items and silently skip rows 32..63
   if (rows == 64 && !(D == 128 && variant == 2 && G == 4)) return -2;
@@ -1431,9 +1444,11 @@ OME_API int ome_paged_prefill_split(const void* q, int64_t q_stride, const void*
                                     const int* items4, int n_items, const int* comb, int n_comb, int chunk,
                                     void* part_o, void* part_ml, void* out, int64_t out_stride, int Hq, int Hkv,
                                     float scale, int window, int kv_fmt, float k_scale, float v_scale, float softcap,
-                                    const float* sinks, const float* alibi, int64_t bsparse, hipStream_t stream) {
+                                    const float* sinks, const float* alibi, int64_t bsparse, int keep_first,
+                                    hipStream_t stream) {
   if (n_items <= 0) return 0;
   if (Hq != 4 * Hkv || chunk % 64 || kv_fmt < 0 || kv_fmt > 2) return -2;
+  if (window > 0 && keep_first > 0) return -6;   // kept first keys: ome_paged_prefill only
   const Scaler scl = make_scaler(scale * k_scale, softcap, alibi, bsparse);
   dim3 grid(n_items, Hkv);
 #define OME_PFS(F, FAST)                                                                                       \

@@ -12,7 +12,7 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 
 template <int ACT>
 __global__ __launch_bounds__(256) void act_and_mul_kernel(const bf16* __restrict__ x, bf16* __restrict__ out,
-                                                          int64_t rows, int I, bool il) {
+                                                          int64_t rows, int I, bool il, float limit) {
   // grid (column blocks, rows): no per-element 64-bit division, every lane one 16-B vector.
   // il: gate / up columns interleaved in 16-column blocks (the layout of a gate_up weight
   // interleaved for the fused SiLU*mul GEMM epilogue, ops.interleave_gate_up)
@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void act_and_mul_kernel(const bf16* __restrict
     if constexpr (ACT == 2 || ACT == 3) {
       // clamped SwiGLU / GeGELU: (clamp(u, -L, L) + 1) * g' * sigmoid(1.702 g'), g' = min(g, L);
       // L = 7 (GPT-OSS), 20 (Phi-3-small gegelu_limit)
-      constexpr float L = ACT == 2 ? 7.f : 20.f;
+      const float L = limit > 0.f ? limit : (ACT == 2 ? 7.f : 20.f);
       const float g2 = fminf(gf, L);
       const float u2 = fminf(fmaxf((float)u[j], -L), L);
       o[j] = (bf16)((u2 + 1.f) * g2 / (1.f + __expf(-1.702f * g2)));
@@ -68,26 +68,62 @@ static inline int grid_for(int64_t work, int nt) {
   return (int)g;
 }
 
-// act: 0 SiLU, 1 GELU-tanh, 2 GPT-OSS clamped SwiGLU (limit 7), 3 Phi-3-small GeGELU (limit 20);
-// | 16: interleaved gate/up (16-col blocks)
-OME_API int ome_act_and_mul(const void* x, void* out, int64_t rows, int I, int act, hipStream_t stream) {
+// Any width (no vector loads): the gated activations for an intermediate size that is not a
+// multiple of 8.  x [rows, 2I] = [gate | up].
+template <typename T>
+__global__ __launch_bounds__(256) void act_and_mul_any_kernel(const T* __restrict__ x, T* __restrict__ out,
+                                                              int I, int act, float limit) {
+  const int64_t r = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= I) return;
+  const float gf = (float)x[r * 2 * I + c], uf = (float)x[r * 2 * I + I + c];
+  float o;
+  if (act == 2 || act == 3) {
+    const float L = limit > 0.f ? limit : (act == 2 ? 7.f : 20.f);
+    const float g2 = fminf(gf, L), u2 = fminf(fmaxf(uf, -L), L);
+    o = (u2 + 1.f) * g2 / (1.f + expf(-1.702f * g2));
+  } else {
+    o = (act == 0 ? silu(gf) : gelu_tanh(gf)) * uf;
+  }
+  out[r * I + c] = (T)o;
+}
+
+// act: 0 SiLU, 1 GELU-tanh, 2 clamped SwiGLU (GPT-OSS: limit 7), 3 Phi-3-small GeGELU (limit 20);
+// limit > 0 replaces the clamp of act 2 / 3; | 16: interleaved gate/up (16-col blocks)
+OME_API int ome_act_and_mul(const void* x, void* out, int64_t rows, int I, int act, float limit,
+                            hipStream_t stream) {
   if (rows <= 0) return 0;
-  const bool il = (act & 16) != 0;
+  const bool il = (act & 16) != 0, f32 = (act & 32) != 0;   // | 32: fp32 elements
   act &= 15;
-  if (I % 8 || (il && I % 16)) return -2;
+  if (il && I % 16) return -2;
+  if (I % 8 || f32) {
+    if (il) return -2;
+    for (int64_t r0 = 0; r0 < rows; r0 += 65535) {
+      const int64_t n = rows - r0 < 65535 ? rows - r0 : 65535;
+      const dim3 g((I + 255) / 256, (unsigned)n);
+      if (f32)
+        act_and_mul_any_kernel<float><<<g, 256, 0, stream>>>((const float*)x + r0 * 2 * I, (float*)out + r0 * I, I,
+                                                             act, limit);
+      else
+        act_and_mul_any_kernel<bf16><<<g, 256, 0, stream>>>((const bf16*)x + r0 * 2 * I, (bf16*)out + r0 * I, I,
+                                                            act, limit);
+    }
+    OME_CHECK_LAUNCH();
+    return 0;
+  }
   for (int64_t r0 = 0; r0 < rows; r0 += 65535) {  // grid.y limit
     const int64_t n = rows - r0 < 65535 ? rows - r0 : 65535;
     const dim3 g((I / 8 + 255) / 256, (unsigned)n);
     const bf16* xp = (const bf16*)x + r0 * 2 * I;
     bf16* op = (bf16*)out + r0 * I;
     if (act == 0)
-      act_and_mul_kernel<0><<<g, 256, 0, stream>>>(xp, op, n, I, il);
+      act_and_mul_kernel<0><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit);
     else if (act == 1)
-      act_and_mul_kernel<1><<<g, 256, 0, stream>>>(xp, op, n, I, il);
+      act_and_mul_kernel<1><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit);
     else if (act == 2)
-      act_and_mul_kernel<2><<<g, 256, 0, stream>>>(xp, op, n, I, il);
+      act_and_mul_kernel<2><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit);
     else
-      act_and_mul_kernel<3><<<g, 256, 0, stream>>>(xp, op, n, I, il);
+      act_and_mul_kernel<3><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit);
   }
   OME_CHECK_LAUNCH();
   return 0;
@@ -222,4 +258,56 @@ OME_API int ome_copy_mapped(const void* src, void* dst, int64_t nbytes, hipStrea
 // Device address of a pinned host allocation (identity on ROCm for hipHostMalloc memory).
 OME_API int ome_host_device_ptr(void* host, void** dev) {
   return hipHostGetDevicePointer(dev, host, 0) == hipSuccess ? 0 : -1;
+}
+
+
+// fp32 rows table[ids] * scale: the start of an fp32 residual stream (ids outside [0, V): zeros)
+template <typename T>
+__global__ __launch_bounds__(256) void embedding_f32_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                                            float* __restrict__ out, int H, int V, float scale) {
+  const int64_t t = blockIdx.x;
+  const int id = ids[t];
+  const bool ok = id >= 0 && id < V;
+  const T* row = table + (int64_t)(ok ? id : 0) * H;
+  for (int i = threadIdx.x; i < H; i += 256) out[t * H + i] = ok ? (float)row[i] * scale : 0.f;
+}
+
+OME_API int ome_embedding_f32(const int* ids, const void* table, float* out, int T, int H, int V, float scale,
+                              int f32, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (f32) embedding_f32_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, H, V, scale);
+  else embedding_f32_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, out, H, V, scale);
+  OME_CHECK_LAUNCH();
+  return 0;
+}
+
+// Output gate of an attention layer: out[t, h * vdim + d] = o[t, h, d] * gate(g[t, h * vdim + d]),
+// d < vdim <= D (o's head rows are D wide; the padding beyond vdim is dropped).  kind 0: sigmoid,
+// 1: SiLU.
+template <typename T>
+__global__ __launch_bounds__(256) void head_gate_kernel(const T* __restrict__ o, const T* __restrict__ g,
+                                                        int64_t g_stride, T* __restrict__ out, int H, int D,
+                                                        int vdim, int kind) {
+  const int64_t t = blockIdx.x;
+  const int n = H * vdim;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const int h = i / vdim, d = i - h * vdim;
+    const float gv = (float)g[t * g_stride + i];
+    const float sg = 1.f / (1.f + expf(-gv));
+    out[t * n + i] = (T)((float)o[(t * H + h) * D + d] * (kind == 0 ? sg : gv * sg));
+  }
+}
+
+OME_API int ome_head_gate(const void* o, const void* g, int64_t g_stride, void* out, int T, int H, int D, int vdim,
+                          int kind, int f32, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (vdim <= 0 || vdim > D) return -2;
+  if (f32)
+    head_gate_kernel<float><<<T, 256, 0, stream>>>((const float*)o, (const float*)g, g_stride, (float*)out, H, D, vdim,
+                                                   kind);
+  else
+    head_gate_kernel<bf16><<<T, 256, 0, stream>>>((const bf16*)o, (const bf16*)g, g_stride, (bf16*)out, H, D, vdim,
+                                                  kind);
+  OME_CHECK_LAUNCH();
+  return 0;
 }

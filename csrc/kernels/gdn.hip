@@ -263,6 +263,81 @@ __global__ __launch_bounds__(256) void gdn_scan_v3_kernel(
     }
 }
 
+
+// Any head shape (dk, dv): the fallback of the kernels above, which need dk in {64, 128, 256}.
+// One workgroup per (sequence, value head); S^T [dv][dk] sits in LDS ([dv][dk + 1]; in global
+// memory when it does not fit) for the whole sequence.  Per row the block forms the unit-norm q
+// (times dk^-1/2) and k of the head's key head in LDS, then thread j runs column j of the state:
+//   S_j <- g S_j;  u = beta (v_j - S_j . k);  S_j <- S_j + u k;  o_j = S_j . q.
+template <typename T>
+__global__ __launch_bounds__(128) void gdn_scan_any_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, int64_t qkv_stride,
+    const T* __restrict__ a, const T* __restrict__ b, int64_t ab_stride, const float* __restrict__ A_log,
+    const float* __restrict__ dt_bias, float* __restrict__ state, T* __restrict__ out, int64_t out_stride,
+    const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ reset, int Hv, int Hk, int dk,
+    int dv, int use_lds) {
+  extern __shared__ float sm[];
+  __shared__ float red[2][2];
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int r0 = cu[s], r1 = cu[s + 1];
+  if (r1 <= r0) return;
+  const int hk = h / (Hv / Hk);
+  float* qs = sm;            // [dk]
+  float* ks = sm + dk;       // [dk]
+  float* gst = state + ((int64_t)slot[s] * Hv + h) * dk * dv;
+  float* st = use_lds ? sm + 2 * dk : gst;
+  const int ld = use_lds ? dk + 1 : dk;
+  const bool fresh = reset[s] != 0;
+  if (use_lds || fresh)
+    for (int e = tid; e < dk * dv; e += 128) st[(e / dk) * ld + e % dk] = fresh ? 0.f : gst[e];
+  const float negA = -expf(A_log[h]), dtb = dt_bias[h];
+  const float qscale = 1.f / sqrtf((float)dk);
+  for (int r = r0; r < r1; ++r) {
+    __syncthreads();   // the previous row's readers of qs / ks are done (and the state is loaded)
+    float sq = 0.f, sk = 0.f;
+    for (int i = tid; i < dk; i += 128) {
+      const float qv = (float)q[(int64_t)r * qkv_stride + (int64_t)hk * dk + i];
+      const float kv = (float)k[(int64_t)r * qkv_stride + (int64_t)hk * dk + i];
+      qs[i] = qv;
+      ks[i] = kv;
+      sq += qv * qv;
+      sk += kv * kv;
+    }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    if ((tid & 63) == 0) {
+      red[tid >> 6][0] = sq;
+      red[tid >> 6][1] = sk;
+    }
+    __syncthreads();
+    const float iq = qscale / sqrtf(red[0][0] + red[1][0] + 1e-6f), ik = 1.f / sqrtf(red[0][1] + red[1][1] + 1e-6f);
+    const float av = (float)a[(int64_t)r * ab_stride + h], bv = (float)b[(int64_t)r * ab_stride + h];
+    const float sp = av + dtb > 20.f ? av + dtb : log1pf(expf(av + dtb));
+    const float decay = expf(negA * sp);
+    const float beta = 1.f / (1.f + expf(-bv));
+    for (int j = tid; j < dv; j += 128) {
+      float* col = st + (int64_t)j * ld;
+      float kv = 0.f;
+      for (int i = 0; i < dk; ++i) {
+        const float sv = col[i] * decay;
+        col[i] = sv;
+        kv += sv * ks[i];
+      }
+      const float u = beta * ((float)v[(int64_t)r * qkv_stride + (int64_t)h * dv + j] - kv * ik);
+      float o = 0.f;
+      for (int i = 0; i < dk; ++i) {
+        const float sv = col[i] + ks[i] * ik * u;
+        col[i] = sv;
+        o += sv * qs[i];
+      }
+      out[(int64_t)r * out_stride + (int64_t)h * dv + j] = (T)(o * iq);
+    }
+  }
+  __syncthreads();
+  if (use_lds)
+    for (int e = tid; e < dk * dv; e += 128) gst[e] = st[(e / dk) * ld + e % dk];
+}
+
 }  // namespace
 
 // q / k / v: row-major views (shared row stride qkv_stride, in elements) of the conv output,
@@ -273,12 +348,27 @@ __global__ __launch_bounds__(256) void gdn_scan_v3_kernel(
 OME_API int ome_gdn_scan(const void* q, const void* k, const void* v, int64_t qkv_stride, const void* a,
                          const void* b, int64_t ab_stride, const float* A_log, const float* dt_bias, float* state,
                          void* out, int64_t out_stride, const int* cu, const int* slot, const int* reset, int S,
-                         int T, int Hv, int Hk, int dk, int dv, float* ws, hipStream_t stream) {
+                         int T, int Hv, int Hk, int dk, int dv, float* ws, int f32, hipStream_t stream) {
   if (S <= 0) return 0;
   if (dv <= 0 || Hk <= 0 || Hv % Hk != 0) return -2;
   static const int nc_env = getenv("OME_GDN_NC") ? atoi(getenv("OME_GDN_NC")) : 0;   // bench override
+  if ((dk != 256 && dk != 128 && dk != 64) || f32) {   // any other key width, fp32 models: the generic kernel
+    if (dk <= 0) return -3;
+    const size_t need = ((size_t)2 * dk + (size_t)dv * (dk + 1)) * sizeof(float);
+    const int use_lds = need <= 60 * 1024;
+    const size_t lds = use_lds ? need : 2 * dk * sizeof(float);
+    if (f32)
+      gdn_scan_any_kernel<float><<<dim3(S, Hv), 128, lds, stream>>>(
+          (const float*)q, (const float*)k, (const float*)v, qkv_stride, (const float*)a, (const float*)b, ab_stride,
+          A_log, dt_bias, state, (float*)out, out_stride, cu, slot, reset, Hv, Hk, dk, dv, use_lds);
+    else
+      gdn_scan_any_kernel<bf16><<<dim3(S, Hv), 128, lds, stream>>>(
+          (const bf16*)q, (const bf16*)k, (const bf16*)v, qkv_stride, (const bf16*)a, (const bf16*)b, ab_stride,
+          A_log, dt_bias, state, (bf16*)out, out_stride, cu, slot, reset, Hv, Hk, dk, dv, use_lds);
+    OME_CHECK_LAUNCH();
+    return 0;
+  }
   if (ws) {   // v3: prep (parallel over rows) + scan; any dv (grid z tiles the state columns)
-    if (dk != 256 && dk != 128 && dk != 64) return -3;
     float* qn = ws;
     float* kn = qn + (int64_t)T * Hk * dk;
     float* qk = kn + (int64_t)T * Hk * dk;

@@ -314,3 +314,56 @@ OME_API int ome_qk_norm_rope(const void* x, int64_t xs, const void* w, const flo
   OME_CHECK_LAUNCH();
   return 0;
 }
+
+
+// ---- fp32 residual stream (decoders that keep x in fp32 for the whole stack) ----
+// res[row] += s1 * x1[row] + s2 * x2[row] (either addend may be null: the outputs of the previous
+// block's sublayer(s), bf16), stored back as fp32, then out[row] = bf16(res * rsqrt(mean(res^2)
+// + eps) * w).  One 256-thread workgroup per row, any width: the sum is formed and written in
+// pass one (with the square sum), pass two re-reads the row it just wrote (cache-hot).
+// T: element type of the addends, the weight and the output (bf16, or float for fp32 models).
+template <typename T>
+__global__ __launch_bounds__(256) void residual_rmsnorm_kernel(float* __restrict__ res, int64_t res_stride,
+                                                               const T* __restrict__ x1, int64_t x1_stride,
+                                                               float s1, const T* __restrict__ x2,
+                                                               int64_t x2_stride, float s2,
+                                                               const T* __restrict__ w, T* __restrict__ out,
+                                                               int64_t out_stride, int H, float eps) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  float* r = res + row * res_stride;
+  const T* a = x1 != nullptr ? x1 + row * x1_stride : nullptr;
+  const T* b = x2 != nullptr ? x2 + row * x2_stride : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    float v = r[i];
+    if (a != nullptr) {
+      float add = s1 * (float)a[i];
+      if (b != nullptr) add += s2 * (float)b[i];
+      v += add;
+      r[i] = v;
+    }
+    ss += v * v;
+  }
+  const float tot = block_sum<256>(ss, red);
+  const float rs = 1.f / sqrtf(tot / (float)H + eps);
+  T* o = out + row * out_stride;
+  for (int i = threadIdx.x; i < H; i += 256) o[i] = (T)(r[i] * rs * (float)w[i]);
+}
+
+OME_API int ome_residual_rmsnorm(float* res, int64_t res_stride, const void* x1, int64_t x1_stride, float s1,
+                                 const void* x2, int64_t x2_stride, float s2, const void* w, void* out,
+                                 int64_t out_stride, int rows, int H, float eps, int f32, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0 || (x1 == nullptr && x2 != nullptr)) return -2;
+  if (f32)
+    residual_rmsnorm_kernel<float><<<rows, 256, 0, stream>>>(res, res_stride, (const float*)x1, x1_stride, s1,
+                                                             (const float*)x2, x2_stride, s2, (const float*)w,
+                                                             (float*)out, out_stride, H, eps);
+  else
+    residual_rmsnorm_kernel<bf16><<<rows, 256, 0, stream>>>(res, res_stride, (const bf16*)x1, x1_stride, s1,
+                                                            (const bf16*)x2, x2_stride, s2, (const bf16*)w,
+                                                            (bf16*)out, out_stride, H, eps);
+  OME_CHECK_LAUNCH();
+  return 0;
+}

@@ -231,3 +231,211 @@ OME_API int ome_kv_cache_write(const void* k, const void* v, int64_t kv_stride, 
   OME_CHECK_LAUNCH();
   return 0;
 }
+
+
+// ---- projection-wide q / k RMSNorm + partial rotary + paged write, any head width <= D ----
+// One 256-thread workgroup per token.  q [Hq*dim] and k [Hkv*dim] are each normalised by ONE root
+// mean square over the whole projection row (weights of that width; null = no norm), then the
+// first rot_dim dims of every head are rotated (interleaved: dim 2i with 2i+1; else i with
+// i + rot_dim/2) by the angle row cos_sin[pos] = [cos(rot_dim/2) | sin(rot_dim/2)], all in fp32
+// with one rounding to bf16 at the store.  Heads are written D wide (q_out [T, Hq, D], K cache
+// [page, Hkv, P, D], V cache [page, Hkv, D, P]) with zeros beyond dim / vdim.
+template <typename T>
+__global__ __launch_bounds__(256) void wide_norm_rope_cache_kernel(
+    const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k, int64_t k_stride,
+    const T* __restrict__ v, int64_t v_stride, const int* __restrict__ positions,
+    const float* __restrict__ cos_sin, int rot_dim, int interleaved, const T* __restrict__ qn_w,
+    const T* __restrict__ kn_w, float eps, T* __restrict__ q_out, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P) {
+  __shared__ float red[4];
+  const int64_t t = blockIdx.x;
+  const T* qr = q + t * q_stride;
+  const T* kr = k + t * k_stride;
+  const T* vr = v + t * v_stride;
+  const int nq = Hq * dim, nk = Hkv * dim;
+  float rq = 1.f, rk = 1.f;
+  if (qn_w != nullptr) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < nq; i += 256) ss += (float)qr[i] * (float)qr[i];
+    rq = 1.f / sqrtf(block_sum<256>(ss, red) / (float)nq + eps);
+  }
+  if (kn_w != nullptr) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < nk; i += 256) ss += (float)kr[i] * (float)kr[i];
+    rk = 1.f / sqrtf(block_sum<256>(ss, red) / (float)nk + eps);
+  }
+  const int half = rot_dim >> 1;
+  const float* cs = cos_sin + (int64_t)positions[t] * rot_dim;
+  const int slot = slots[t];
+  const int64_t page = slot >= 0 ? slot / P : 0, off = slot >= 0 ? slot % P : 0;
+  const int hp = D >> 1;   // dim pairs per (padded) head
+  // q and k: one unit = one pair of dims of one head
+  for (int u = threadIdx.x; u < (Hq + Hkv) * hp; u += 256) {
+    const int h = u / hp, j = u - h * hp;
+    const bool is_q = h < Hq;
+    const int hh = is_q ? h : h - Hq;
+    int d0, d1;
+    if (j < half) {
+      d0 = interleaved ? 2 * j : j;
+      d1 = interleaved ? 2 * j + 1 : j + half;
+    } else {
+      d0 = rot_dim + 2 * (j - half);
+      d1 = d0 + 1;
+    }
+    const T* src = is_q ? qr : kr;
+    const T* nw = is_q ? qn_w : kn_w;
+    const float rs = is_q ? rq : rk;
+    float a = 0.f, b = 0.f;
+    if (d0 < dim) {
+      a = (float)src[hh * dim + d0];
+      if (nw != nullptr) a = a * rs * (float)nw[hh * dim + d0];
+    }
+    if (d1 < dim) {
+      b = (float)src[hh * dim + d1];
+      if (nw != nullptr) b = b * rs * (float)nw[hh * dim + d1];
+    }
+    if (j < half) {
+      const float c = cs[j], sn = cs[half + j];
+      const float ra = a * c - b * sn, rb = b * c + a * sn;
+      a = ra;
+      b = rb;
+    }
+    if (is_q) {
+      T* dst = q_out + (t * Hq + hh) * D;
+      if (d0 < D) dst[d0] = (T)a;
+      if (d1 < D) dst[d1] = (T)b;
+    } else if (slot >= 0) {
+      T* dst = k_cache + ((page * Hkv + hh) * P + off) * D;
+      if (d0 < D) dst[d0] = (T)a;
+      if (d1 < D) dst[d1] = (T)b;
+    }
+  }
+  // v: transposed scatter [page][kh][d][off], zeros beyond vdim
+  if (slot >= 0) {
+    for (int i = threadIdx.x; i < Hkv * D; i += 256) {
+      const int kh = i / D, d = i - kh * D;
+      const float x = d < vdim ? (float)vr[kh * vdim + d] : 0.f;
+      v_cache[((page * Hkv + kh) * D + d) * P + off] = (T)x;
+    }
+  }
+}
+
+// The same op with 16-byte accesses, for the shapes real layers have: interleaved rotation (a
+// pair never leaves its 8-wide vector), dim % 8 == 0, rows and pointers 16-byte aligned.  A unit
+// is one 8-dim vector of one head; pass one sums the squares from vector loads, pass two re-reads
+// the (cache-hot) row, normalises, rotates in registers and stores one vector.
+__global__ __launch_bounds__(256) void wide_norm_rope_cache_vec_kernel(
+    const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k, int64_t k_stride,
+    const bf16* __restrict__ v, int64_t v_stride, const int* __restrict__ positions,
+    const float* __restrict__ cos_sin, int rot_dim, const bf16* __restrict__ qn_w, const bf16* __restrict__ kn_w,
+    float eps, bf16* __restrict__ q_out, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
+    const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P) {
+  __shared__ float red[4];
+  const int64_t t = blockIdx.x;
+  const bf16* qr = q + t * q_stride;
+  const bf16* kr = k + t * k_stride;
+  const bf16* vr = v + t * v_stride;
+  const int nq = Hq * dim, nk = Hkv * dim;
+  float rq = 1.f, rk = 1.f;
+  if (qn_w != nullptr) {
+    float ss = 0.f;
+    for (int i = threadIdx.x * 8; i < nq; i += 2048) {
+      const bf16x8 x = ld8(qr + i);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += (float)x[j] * (float)x[j];
+    }
+    rq = 1.f / sqrtf(block_sum<256>(ss, red) / (float)nq + eps);
+  }
+  if (kn_w != nullptr) {
+    float ss = 0.f;
+    for (int i = threadIdx.x * 8; i < nk; i += 2048) {
+      const bf16x8 x = ld8(kr + i);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += (float)x[j] * (float)x[j];
+    }
+    rk = 1.f / sqrtf(block_sum<256>(ss, red) / (float)nk + eps);
+  }
+  const int half = rot_dim >> 1;
+  const float* cs = cos_sin + (int64_t)positions[t] * rot_dim;
+  const int slot = slots[t];
+  const int64_t page = slot >= 0 ? slot / P : 0, off = slot >= 0 ? slot % P : 0;
+  const int vph = D >> 3;   // vectors per (padded) head
+  for (int u = threadIdx.x; u < (Hq + Hkv) * vph; u += 256) {
+    const int h = u / vph, d0 = (u - h * vph) * 8;
+    const bool is_q = h < Hq;
+    const int hh = is_q ? h : h - Hq;
+    if (!is_q && slot < 0) continue;
+    bf16x8 o = {};
+    if (d0 < dim) {
+      const bf16* src = (is_q ? qr : kr) + hh * dim + d0;
+      const bf16* nw = is_q ? qn_w : kn_w;
+      const bf16x8 x = ld8(src);
+      float f[8];
+      if (nw != nullptr) {
+        const bf16x8 wv = ld8(nw + hh * dim + d0);
+        const float rs = is_q ? rq : rk;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] = (float)x[j] * rs * (float)wv[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] = (float)x[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = d0 + 2 * j;
+        if (d < rot_dim) {
+          const float c = cs[d >> 1], sn = cs[half + (d >> 1)];
+          const float a = f[2 * j], b = f[2 * j + 1];
+          f[2 * j] = a * c - b * sn;
+          f[2 * j + 1] = b * c + a * sn;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = (bf16)f[j];
+    }
+    if (is_q) st8(q_out + (t * Hq + hh) * D + d0, o);
+    else st8(k_cache + ((page * Hkv + hh) * P + off) * D + d0, o);
+  }
+  if (slot >= 0) {   // v: lanes take consecutive dims (rows 2 * P bytes apart), zeros beyond vdim
+    for (int i = threadIdx.x; i < Hkv * D; i += 256) {
+      const int kh = i / D, d = i - kh * D;
+      v_cache[((page * Hkv + kh) * D + d) * P + off] = d < vdim ? vr[kh * vdim + d] : (bf16)0.f;
+    }
+  }
+}
+
+OME_API int ome_wide_norm_rope_cache(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                                     int64_t v_stride, const int* positions, const float* cos_sin, int rot_dim,
+                                     int interleaved, const void* qn_w, const void* kn_w, float eps, void* q_out,
+                                     void* k_cache, void* v_cache, const int* slots, int T, int Hq, int Hkv, int dim,
+                                     int vdim, int D, int P, int f32, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (dim <= 0 || vdim <= 0 || dim > D || vdim > D || (D & 1) || rot_dim < 0 || rot_dim > dim || (rot_dim & 1))
+    return -2;
+  if (f32) {   // fp32 model: fp32 projections, norm weights, q and cache
+    wide_norm_rope_cache_kernel<float><<<T, 256, 0, stream>>>(
+        (const float*)q, q_stride, (const float*)k, k_stride, (const float*)v, v_stride, positions, cos_sin, rot_dim,
+        interleaved, (const float*)qn_w, (const float*)kn_w, eps, (float*)q_out, (float*)k_cache, (float*)v_cache,
+        slots, Hq, Hkv, dim, vdim, D, P);
+    OME_CHECK_LAUNCH();
+    return 0;
+  }
+  const bool vec = interleaved && dim % 8 == 0 && D % 8 == 0 && q_stride % 8 == 0 && k_stride % 8 == 0 &&
+                   (uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)q_out % 16 == 0 &&
+                   (uintptr_t)k_cache % 16 == 0 && (qn_w == nullptr || (uintptr_t)qn_w % 16 == 0) &&
+                   (kn_w == nullptr || (uintptr_t)kn_w % 16 == 0);
+  if (vec) {
+    wide_norm_rope_cache_vec_kernel<<<T, 256, 0, stream>>>(
+        (const bf16*)q, q_stride, (const bf16*)k, k_stride, (const bf16*)v, v_stride, positions, cos_sin, rot_dim,
+        (const bf16*)qn_w, (const bf16*)kn_w, eps, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, slots, Hq, Hkv, dim,
+        vdim, D, P);
+    OME_CHECK_LAUNCH();
+    return 0;
+  }
+  wide_norm_rope_cache_kernel<bf16><<<T, 256, 0, stream>>>(
+      (const bf16*)q, q_stride, (const bf16*)k, k_stride, (const bf16*)v, v_stride, positions, cos_sin, rot_dim,
+      interleaved, (const bf16*)qn_w, (const bf16*)kn_w, eps, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, slots,
+      Hq, Hkv, dim, vdim, D, P);
+  OME_CHECK_LAUNCH();
+  return 0;
+}

@@ -179,40 +179,131 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
   }
 }
 
-__global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const bf16* __restrict__ y, int64_t y_stride,
-                                                            const bf16* __restrict__ z, int64_t z_stride,
-                                                            const bf16* __restrict__ w, bf16* __restrict__ out,
+// T = float (fp32 models): no intermediate rounding; bf16: the normalised value is rounded before
+// the scale, as the reference implementations of the bf16 families do.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const T* __restrict__ y, int64_t y_stride,
+                                                            const T* __restrict__ z, int64_t z_stride,
+                                                            const T* __restrict__ w, T* __restrict__ out,
                                                             int64_t out_stride, int group, float eps, int norm_first) {
   __shared__ float red[4];
   const int row = blockIdx.y, g0 = blockIdx.x * group;
-  const bf16* yr = y + (int64_t)row * y_stride + g0;
-  const bf16* zr = z + (int64_t)row * z_stride + g0;
+  const T* yr = y + (int64_t)row * y_stride + g0;
+  const T* zr = z + (int64_t)row * z_stride + g0;
   float ss = 0.f;
   for (int i = threadIdx.x; i < group; i += 256) {
     const float v = norm_first ? (float)yr[i] : (float)yr[i] * silu_f((float)zr[i]);
     ss += v * v;
   }
   const float tot = block_sum<256>(ss, red);
-  const float rs = rsqrtf(tot / (float)group + eps);
-  bf16* orow = out + (int64_t)row * out_stride + g0;
+  const float rs = 1.f / sqrtf(tot / (float)group + eps);
+  T* orow = out + (int64_t)row * out_stride + g0;
   for (int i = threadIdx.x; i < group; i += 256) {
     if (norm_first) {   // Qwen3-Next: w (per group channel) * norm(y), then * silu(z)
-      const float t = (float)(bf16)((float)(bf16)((float)yr[i] * rs) * (float)w[i]);
-      orow[i] = (bf16)(t * silu_f((float)zr[i]));
+      const float t = (float)(T)((float)(T)((float)yr[i] * rs) * (float)w[i]);
+      orow[i] = (T)(t * silu_f((float)zr[i]));
     } else {
       const float v = (float)yr[i] * silu_f((float)zr[i]) * rs;
-      orow[i] = (bf16)((float)(bf16)v * (float)w[g0 + i]);  // HF: normalise, cast, then scale by w
+      orow[i] = (T)((float)(T)v * (float)w[g0 + i]);  // HF: normalise, cast, then scale by w
     }
   }
+}
+
+
+// Any tap count 1 <= K <= 16 (the templated kernels cover 2..6): same arguments, runtime loops.
+template <typename T>
+__global__ __launch_bounds__(256) void ssm_conv1d_any_kernel(const T* __restrict__ x, int64_t x_stride,
+                                                             const T* __restrict__ w, const T* __restrict__ bias,
+                                                             T* __restrict__ out, int64_t out_stride,
+                                                             T* __restrict__ state, const int* __restrict__ cu,
+                                                             const int* __restrict__ slot, const int* __restrict__ reset,
+                                                             int C, int K) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int s = blockIdx.y;
+  if (c >= C) return;
+  const int r0 = cu[s], r1 = cu[s + 1];
+  if (r1 <= r0) return;
+  T* st = state + ((int64_t)slot[s] * C + c) * (K - 1);
+  float win[15], wt[16];
+  const bool fresh = reset[s] != 0;
+  for (int j = 0; j < K - 1; ++j) win[j] = fresh ? 0.f : (float)st[j];
+  for (int j = 0; j < K; ++j) wt[j] = (float)w[(int64_t)c * K + j];
+  const float b = bias != nullptr ? (float)bias[c] : 0.f;
+  for (int r = r0; r < r1; ++r) {
+    const float v = (float)x[(int64_t)r * x_stride + c];
+    float acc = b + wt[K - 1] * v;
+    for (int j = 0; j < K - 1; ++j) acc += wt[j] * win[j];
+    for (int j = 0; j + 1 < K - 1; ++j) win[j] = win[j + 1];
+    if (K > 1) win[K - 2] = v;
+    out[(int64_t)r * out_stride + c] = (T)(acc / (1.f + expf(-acc)));
+  }
+  for (int j = 0; j < K - 1; ++j) st[j] = (T)win[j];
+}
+
+// Any head shape (P x N) and unaligned operand views: the fallback of ssm_scan_kernel, which needs
+// 256 % P == 0, N / (256 / P) in {8, 16, 32, 64} and 16-byte aligned B / C rows.  One workgroup
+// per (head, sequence); the head's fp32 state lives in LDS ([P][N + 1], or stays in global memory
+// when it does not fit) for the whole sequence; per row: every thread updates its share of the
+// P x N entries, then thread p reduces row p against C.  Two barriers per row.
+template <typename T>
+__global__ __launch_bounds__(256) void ssm_scan_any_kernel(
+    const T* __restrict__ x, int64_t x_stride, const T* __restrict__ dt, int64_t dt_stride,
+    const T* __restrict__ B, const T* __restrict__ Cm, int64_t bc_stride, const float* __restrict__ A,
+    const float* __restrict__ D, const float* __restrict__ dt_bias, float dt_min, float* __restrict__ state,
+    T* __restrict__ y, int64_t y_stride, const int* __restrict__ cu, const int* __restrict__ slot,
+    const int* __restrict__ reset, int H, int P, int N, int G, int use_lds) {
+  extern __shared__ float sm[];
+  const int h = blockIdx.x, s = blockIdx.y;
+  const int r0 = cu[s], r1 = cu[s + 1];
+  if (r1 <= r0) return;
+  const int g = h / (H / G);
+  float* gst = state + ((int64_t)slot[s] * H + h) * P * N;
+  float* st = use_lds ? sm : gst;
+  const int ld = use_lds ? N + 1 : N;
+  const int PN = P * N;
+  const bool fresh = reset[s] != 0;
+  if (use_lds || fresh)
+    for (int e = threadIdx.x; e < PN; e += 256) st[(e / N) * ld + e % N] = fresh ? 0.f : gst[e];
+  __syncthreads();
+  const float a = A[h], d = D[h], db = dt_bias[h];
+  for (int r = r0; r < r1; ++r) {
+    const float dtr = (float)dt[(int64_t)r * dt_stride + h] + db;
+    const float dtv = fmaxf(dtr > 20.f ? dtr : log1pf(expf(dtr)), dt_min);
+    const float dA = expf(dtv * a);
+    const T* xr = x + (int64_t)r * x_stride + h * P;
+    const T* br = B + (int64_t)r * bc_stride + (int64_t)g * N;
+    const T* cr = Cm + (int64_t)r * bc_stride + (int64_t)g * N;
+    for (int e = threadIdx.x; e < PN; e += 256) {
+      const int p = e / N, n = e - p * N;
+      st[p * ld + n] = st[p * ld + n] * dA + dtv * (float)xr[p] * (float)br[n];
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < P; p += 256) {
+      float acc = 0.f;
+      for (int n = 0; n < N; ++n) acc += (float)cr[n] * st[p * ld + n];
+      y[(int64_t)r * y_stride + h * P + p] = (T)(acc + d * (float)xr[p]);
+    }
+    __syncthreads();
+  }
+  if (use_lds)
+    for (int e = threadIdx.x; e < PN; e += 256) gst[e] = st[(e / N) * ld + e % N];
 }
 
 }  // namespace
 
 OME_API int ome_ssm_conv1d(const void* x, int64_t x_stride, const void* w, const void* bias, void* out,
                            int64_t out_stride, void* state, const int* cu, const int* slot, const int* reset, int S,
-                           int C, int K, hipStream_t stream) {
+                           int C, int K, int f32, hipStream_t stream) {
   if (S <= 0 || C <= 0) return 0;
   dim3 grid((C + 255) / 256, S);
+  if (f32) {   // fp32 models: inputs, taps, outputs and the tail state are float
+    if (K < 1 || K > 16) return -2;
+    ssm_conv1d_any_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, (const float*)w,
+                                                           (const float*)bias, (float*)out, out_stride,
+                                                           (float*)state, cu, slot, reset, C, K);
+    OME_CHECK_LAUNCH();
+    return 0;
+  }
 #define CONV_CASE(KK)                                                                                         \
   case KK:                                                                                                     \
     ssm_conv1d_kernel<KK><<<grid, 256, 0, stream>>>((const bf16*)x, x_stride, (const bf16*)w, (const bf16*)bias, \
@@ -225,7 +316,10 @@ OME_API int ome_ssm_conv1d(const void* x, int64_t x_stride, const void* w, const
     CONV_CASE(5)
     CONV_CASE(6)
     default:
-      return -2;
+      if (K < 1 || K > 16) return -2;
+      ssm_conv1d_any_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)x, x_stride, (const bf16*)w, (const bf16*)bias,
+                                                      (bf16*)out, out_stride, (bf16*)state, cu, slot, reset, C, K);
+      break;
   }
 #undef CONV_CASE
   OME_CHECK_LAUNCH();
@@ -260,9 +354,31 @@ OME_API int ome_dyn_conv1d(const void* x, int64_t x_stride, const void* kern, in
 OME_API int ome_ssm_scan(const void* x, int64_t x_stride, const void* dt, int64_t dt_stride, const void* B,
                          const void* Cm, int64_t bc_stride, const float* A, const float* D, const float* dt_bias,
                          float dt_min, float* state, void* y, int64_t y_stride, const int* cu, const int* slot,
-                         const int* reset, int S, int H, int P, int N, int G, hipStream_t stream) {
+                         const int* reset, int S, int H, int P, int N, int G, int f32, hipStream_t stream) {
   if (S <= 0) return 0;
-  if (P <= 0 || 256 % P != 0 || H % G != 0) return -2;
+  if (P <= 0 || N <= 0 || G <= 0 || H % G != 0) return -2;
+  {
+    // the register-resident kernel needs its tiling (256 % P, 8 | N / (256 / P) <= 64) and B / C
+    // rows it can read as 16-byte vectors; every other shape or view takes the generic kernel
+    const int tp = 256 % P == 0 ? 256 / P : 0;
+    const int np = tp > 0 && N % tp == 0 ? N / tp : 0;
+    const bool fast = (np == 8 || np == 16 || np == 32 || np == 64) && bc_stride % 8 == 0 && N % 8 == 0 &&
+                      ((uintptr_t)B % 16 == 0) && ((uintptr_t)Cm % 16 == 0) && ((uintptr_t)state % 16 == 0);
+    if (!fast || f32) {
+      const size_t need = (size_t)P * (N + 1) * sizeof(float);
+      const int use_lds = need <= 64 * 1024;
+      if (f32)
+        ssm_scan_any_kernel<float><<<dim3(H, S), 256, use_lds ? need : 0, stream>>>(
+            (const float*)x, x_stride, (const float*)dt, dt_stride, (const float*)B, (const float*)Cm, bc_stride, A,
+            D, dt_bias, dt_min, state, (float*)y, y_stride, cu, slot, reset, H, P, N, G, use_lds);
+      else
+        ssm_scan_any_kernel<bf16><<<dim3(H, S), 256, use_lds ? need : 0, stream>>>(
+            (const bf16*)x, x_stride, (const bf16*)dt, dt_stride, (const bf16*)B, (const bf16*)Cm, bc_stride, A, D,
+            dt_bias, dt_min, state, (bf16*)y, y_stride, cu, slot, reset, H, P, N, G, use_lds);
+      OME_CHECK_LAUNCH();
+      return 0;
+    }
+  }
   // rows per workgroup: the whole head (PB = P).  Splitting a head's rows over more workgroups
   // (PB = P/4, 8 states per lane) measured SLOWER for 2 x 512-row prefill on gfx950 (812 vs 550 us,
   // scripts/ssm_scan_bench.py): the row loop is latency-bound per step, not occupancy-bound.
@@ -302,13 +418,18 @@ OME_API int ome_ssm_scan(const void* x, int64_t x_stride, const void* dt, int64_
 
 OME_API int ome_gated_rmsnorm(const void* y, int64_t y_stride, const void* z, int64_t z_stride, const void* w,
                               void* out, int64_t out_stride, int rows, int I, int group, float eps,
-                              int norm_first, hipStream_t stream) {
+                              int norm_first, int f32, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (group <= 0 || I % group != 0) return -2;
   dim3 grid(I / group, rows);
-  gated_rmsnorm_kernel<<<grid, 256, 0, stream>>>((const bf16*)y, y_stride, (const bf16*)z, z_stride,
-                                                 (const bf16*)w, (bf16*)out, out_stride, group, eps,
-                                                 norm_first);
+  if (f32)
+    gated_rmsnorm_kernel<float><<<grid, 256, 0, stream>>>((const float*)y, y_stride, (const float*)z, z_stride,
+                                                          (const float*)w, (float*)out, out_stride, group, eps,
+                                                          norm_first);
+  else
+    gated_rmsnorm_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)y, y_stride, (const bf16*)z, z_stride,
+                                                         (const bf16*)w, (bf16*)out, out_stride, group, eps,
+                                                         norm_first);
   OME_CHECK_LAUNCH();
   return 0;
 }

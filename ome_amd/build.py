@@ -37,8 +37,9 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found (ROCm toolchain required to build ome_amd kernels)")
 
 
+# (packed fp32 VALU ops are switched off for every kernel: scalar fp32 code only)
 HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-munsafe-fp-atomics",
-             "-Wno-unused-result"]
+             "-Wno-unused-result", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-pthread", "-Wall", "-Wno-unused-function"]
 
 

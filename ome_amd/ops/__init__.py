@@ -18,6 +18,18 @@ def _gpu(t: torch.Tensor) -> bool:
     return t.is_cuda
 
 
+def _f32(t: torch.Tensor, *same) -> int:
+    """1 when ``t`` (and every tensor of ``same`` that is not None) is float32, 0 when they are all
+    bfloat16 -- the element-type switch of the kernels that serve fp32 models too; anything else
+    (or a mix) raises."""
+    ts = [t] + [x for x in same if x is not None]
+    if all(x.dtype == torch.float32 for x in ts):
+        return 1
+    if all(x.dtype == torch.bfloat16 for x in ts):
+        return 0
+    raise TypeError(f"operands must be all bfloat16 or all float32, got {[str(x.dtype) for x in ts]}")
+
+
 def _i32(t: torch.Tensor) -> torch.Tensor:
     assert t.dtype == torch.int32 and t.is_contiguous(), "metadata tensors must be contiguous int32"
     return t
@@ -123,7 +135,7 @@ def ssm_conv1d(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, stat
     assert x.stride(1) == 1 and out.stride(1) == 1 and w.is_contiguous() and state.is_contiguous()
     call("ome_ssm_conv1d", x.data_ptr(), x.stride(0), w.data_ptr(), ptr(bias), out.data_ptr(), out.stride(0),
          state.data_ptr(), _i32(cu).data_ptr(), _i32(slot).data_ptr(), _i32(reset).data_ptr(), slot.shape[0], C,
-         w.shape[1], stream_ptr())
+         w.shape[1], _f32(x, w, bias, out, state), stream_ptr())
     return out
 
 
@@ -157,7 +169,7 @@ def ssm_scan(x, dt, B, C, A, D, dt_bias, dt_min: float, state, cu, slot, reset, 
     call("ome_ssm_scan", x.data_ptr(), x.stride(0), dt.data_ptr(), dt.stride(0), B.data_ptr(), C.data_ptr(),
          B.stride(0), A.data_ptr(), D.data_ptr(), dt_bias.data_ptr(), float(dt_min), state.data_ptr(),
          out.data_ptr(), out.stride(0), _i32(cu).data_ptr(), _i32(slot).data_ptr(), _i32(reset).data_ptr(),
-         slot.shape[0], H, P, N, G, stream_ptr())
+         slot.shape[0], H, P, N, G, _f32(x, dt, B, C, out), stream_ptr())
     return out
 
 
@@ -175,12 +187,15 @@ def gdn_scan(q, k, v, a, b, A_log, dt_bias, state, cu, slot, reset, Hv: int, Hk:
         return ref.gdn_scan(q, k, v, a, b, A_log, dt_bias, state, cu, slot, reset, Hv, Hk, out)
     assert q.stride(0) == k.stride(0) == v.stride(0) and a.stride(0) == b.stride(0)
     assert q.stride(1) == k.stride(1) == v.stride(1) == a.stride(1) == 1 and out.stride(1) == 1
-    assert state.is_contiguous() and state.dtype == torch.float32 and q.dtype == torch.bfloat16
-    ws = None if v1 else torch.empty(T * (2 * Hk * dk + Hk + 2 * Hv), dtype=torch.float32, device=q.device)
+    assert state.is_contiguous() and state.dtype == torch.float32
+    f32 = _f32(q, k, v, a, b, out)
+    # (key widths other than 64 / 128 / 256, and fp32 models, run the launcher's generic kernel: no workspace)
+    ws = None if v1 or f32 or dk not in (64, 128, 256) else \
+        torch.empty(T * (2 * Hk * dk + Hk + 2 * Hv), dtype=torch.float32, device=q.device)
     call("ome_gdn_scan", q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), a.data_ptr(), b.data_ptr(),
          a.stride(0), A_log.data_ptr(), dt_bias.data_ptr(), state.data_ptr(), out.data_ptr(), out.stride(0),
          _i32(cu).data_ptr(), _i32(slot).data_ptr(), _i32(reset).data_ptr(), slot.shape[0], T, Hv, Hk, dk, dv,
-         ptr(ws), stream_ptr())
+         ptr(ws), f32, stream_ptr())
     return out
 
 
@@ -193,7 +208,7 @@ def gated_rmsnorm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, group: int,
     T, I = y.shape
     out = torch.empty(T, I, dtype=y.dtype, device=y.device)
     call("ome_gated_rmsnorm", y.data_ptr(), y.stride(0), z.data_ptr(), z.stride(0), w.data_ptr(), out.data_ptr(),
-         out.stride(0), T, I, group, float(eps), int(norm_first), stream_ptr())
+         out.stride(0), T, I, group, float(eps), int(norm_first), _f32(y, z, w), stream_ptr())
     return out
 
 
@@ -232,19 +247,22 @@ def kv_cache_write(k, v, k_cache, v_cache, slots, k_scale: float = 1.0, v_scale:
 
 
 def act_and_mul(x: torch.Tensor, act: int = 0, out: torch.Tensor | None = None,
-                interleaved: bool = False) -> torch.Tensor:
+                interleaved: bool = False, limit: float = 0.0) -> torch.Tensor:
     """act 0 = SiLU (SwiGLU), 1 = GELU-tanh (GeGLU), 2 = GPT-OSS clamped SwiGLU, 3 = Phi-3-small
     GeGELU (quick-GELU gate, limit 20, ``up + 1``).  x [.., 2I] -> [.., I].  ``interleaved``:
-    gate / up columns alternate in 16-column blocks (:func:`interleave_gate_up` weights)."""
+    gate / up columns alternate in 16-column blocks (:func:`interleave_gate_up` weights).
+    ``limit`` > 0 replaces the clamp of act 2 / 3 (0: the family's constant)."""
     if not _gpu(x):
         if interleaved:
             g, u = deinterleave_gate_up(x.reshape(-1, x.shape[-1]))
             x = torch.cat([g, u], -1).view(*x.shape)
-        return ref.act_and_mul(x, act)
+        return ref.act_and_mul(x, act, limit)
     I = x.shape[-1] // 2
     rows = x.numel() // x.shape[-1]
+    assert x.is_contiguous()
     out = torch.empty(*x.shape[:-1], I, dtype=x.dtype, device=x.device) if out is None else out
-    call("ome_act_and_mul", x.data_ptr(), out.data_ptr(), rows, I, act | (16 if interleaved else 0), stream_ptr())
+    call("ome_act_and_mul", x.data_ptr(), out.data_ptr(), rows, I,
+         act | (16 if interleaved else 0) | (32 if _f32(x, out) else 0), float(limit), stream_ptr())
     return out
 
 
@@ -258,6 +276,99 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, vocab_start: int = 0, voca
     call("ome_embedding", _i32(ids).data_ptr(), table.data_ptr(), out.data_ptr(), T, H, vocab_start, vocab_end,
          stream_ptr())
     return out
+
+
+def embedding_f32(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """fp32 [T, H] rows ``table[ids] * scale``: the start of an fp32 residual stream."""
+    if not _gpu(ids):
+        return ref.embedding_f32(ids, table, scale)
+    T, H = ids.shape[0], table.shape[1]
+    assert table.is_contiguous()
+    out = torch.empty(T, H, dtype=torch.float32, device=table.device)
+    call("ome_embedding_f32", _i32(ids).data_ptr(), table.data_ptr(), out.data_ptr(), T, H, table.shape[0],
+         float(scale), _f32(table), stream_ptr())
+    return out
+
+
+def residual_rmsnorm(res: torch.Tensor, w: torch.Tensor, eps: float, x1: torch.Tensor | None = None,
+                     s1: float = 1.0, x2: torch.Tensor | None = None, s2: float = 1.0,
+                     out_dtype=None) -> torch.Tensor:
+    """Pre-norm step of an fp32 residual stream: ``res += s1 * x1 + s2 * x2`` in place (the
+    sublayer outputs of the previous block, either may be None; two addends serve blocks with two
+    mixers side by side), then ``rmsnorm(res) * w`` in the model dtype -- sum, mean square and
+    scaling in fp32, one rounding at the end."""
+    if not _gpu(res):
+        return ref.residual_rmsnorm(res, w, eps, x1, s1, x2, s2, out_dtype)
+    T, H = res.shape
+    assert res.dtype == torch.float32 and res.stride(1) == 1
+    if x2 is not None and x1 is None:
+        x1, s1, x2, s2 = x2, s2, None, 1.0
+    for a in (x1, x2):
+        assert a is None or (a.shape == res.shape and a.stride(1) == 1)
+    f32 = _f32(w, x1, x2)
+    out = torch.empty(T, H, dtype=w.dtype, device=res.device)
+    call("ome_residual_rmsnorm", res.data_ptr(), res.stride(0), ptr(x1), x1.stride(0) if x1 is not None else 0,
+         float(s1), ptr(x2), x2.stride(0) if x2 is not None else 0, float(s2), w.data_ptr(), out.data_ptr(),
+         out.stride(0), T, H, float(eps), f32, stream_ptr())
+    return out
+
+
+def wide_norm_rope_cache(q, k, v, positions, cos_sin, rot_dim: int, interleaved: bool, qn_w, kn_w, eps: float,
+                         q_out, k_cache, v_cache, slots, Hq: int, Hkv: int, dim: int, vdim: int) -> None:
+    """q [T, Hq*dim], k [T, Hkv*dim], v [T, Hkv*vdim] (row-strided views of a fused projection) ->
+    projection-wide RMSNorm of q and of k (ONE root mean square over all heads' channels of a row,
+    weights ``qn_w`` / ``kn_w`` of the projection's width, None = no norm), rotary embedding on the
+    first ``rot_dim`` dims of each head (``interleaved``: dim 2i pairs with 2i+1, else i with
+    i + rot_dim/2; angles from the ``cos_sin`` table row of the token's position), q into
+    ``q_out`` [T, Hq, D], k / v into the paged cache at ``slots``.  ``dim`` / ``vdim`` <= D (the
+    cache's head width): the tail of every head is written as zeros, which adds nothing to a score
+    and leaves the padded output columns zero."""
+    P, D = k_cache.shape[2], k_cache.shape[3]
+    assert dim <= D and vdim <= D and rot_dim <= dim and rot_dim % 2 == 0
+    if not _gpu(q):
+        return ref.wide_norm_rope_cache(q, k, v, positions, cos_sin, rot_dim, interleaved, qn_w, kn_w, eps, q_out,
+                                        k_cache, v_cache, slots, Hq, Hkv, dim, vdim, P)
+    f32 = _f32(q, k, v, qn_w, kn_w, q_out, k_cache, v_cache)
+    assert q_out.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert q.stride(1) == k.stride(1) == v.stride(1) == 1 and cos_sin.dtype == torch.float32
+    assert cos_sin.shape[1] == rot_dim or rot_dim == 0
+    call("ome_wide_norm_rope_cache", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+         _i32(positions).data_ptr(), cos_sin.data_ptr(), int(rot_dim), int(bool(interleaved)), ptr(qn_w), ptr(kn_w),
+         float(eps), q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _i32(slots).data_ptr(), q.shape[0],
+         Hq, Hkv, dim, vdim, D, P, f32, stream_ptr())
+
+
+def head_gate(o: torch.Tensor, g: torch.Tensor, vdim: int, kind: int = 0) -> torch.Tensor:
+    """Output gate of an attention layer: ``o`` [T, H, D] (head width possibly padded beyond
+    ``vdim``) times ``sigmoid(g)`` (kind 0) or ``silu(g)`` (kind 1), g a row-strided [T, H*vdim]
+    view -> contiguous [T, H*vdim] (the out-projection's input, padding dropped)."""
+    if not _gpu(o):
+        return ref.head_gate(o, g, vdim, kind)
+    T, H, D = o.shape
+    assert o.is_contiguous() and g.stride(1) == 1
+    out = torch.empty(T, H * vdim, dtype=o.dtype, device=o.device)
+    call("ome_head_gate", o.data_ptr(), g.data_ptr(), g.stride(0), out.data_ptr(), T, H, D, vdim, int(kind),
+         _f32(o, g), stream_ptr())
+    return out
+
+
+_MM_OUT_DTYPE = [None]   # does torch.mm take out_dtype on this build (bf16 x bf16 -> fp32)?
+
+
+def lm_head_f32(hidden: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """fp32 logits ``hidden @ w.T``: 16-bit operands, fp32 accumulation AND fp32 result (no
+    rounding of the logits to the model dtype) -- the library GEMM."""
+    if hidden.dtype == torch.float32 or not _gpu(hidden):
+        return F.linear(hidden.float(), w.float())
+    if _MM_OUT_DTYPE[0] is None:
+        try:
+            torch.mm(hidden[:1], w[:8].t(), out_dtype=torch.float32)
+            _MM_OUT_DTYPE[0] = True
+        except (TypeError, RuntimeError):
+            _MM_OUT_DTYPE[0] = False
+    if _MM_OUT_DTYPE[0]:
+        return torch.mm(hidden, w.t(), out_dtype=torch.float32)
+    return torch.mm(hidden.float(), w.float().t())
 
 
 def fill_pending(ids: torch.Tensor, src: torch.Tensor, prev: torch.Tensor) -> None:
@@ -672,22 +783,29 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, ws: DecodeW
                  window: int = -1, out=None, order: torch.Tensor | None = None, k_scale: float = 1.0,
                  v_scale: float = 1.0, softcap: float = 0.0, sinks: torch.Tensor | None = None,
                  alibi: torch.Tensor | None = None, row_lo: torch.Tensor | None = None,
-                 blocksparse: tuple | None = None) -> torch.Tensor:
+                 blocksparse: tuple | None = None, keep_first: int = 0) -> torch.Tensor:
     """q [B, Hq, D] -> [B, Hq, D].  ``alibi``: fp32 [Hq] ALiBi slopes (logit += slope * (key - query
     position)), or None.  ``row_lo``: int32 [B], row b attends keys [row_lo[b], seq_lens[b]) only
     (Mllama cross attention over a range of a request's vision-token cache).  ``order`` (int32 [B], optional): sequence visit order for the
     workgroup dispatcher (longest first balances the tail).  The cache may be bf16 or fp8
     (``k_scale`` / ``v_scale`` dequantise it).  ``blocksparse``: (block, local_blocks, vert_stride,
-    head_step, head0) block-sparse causal mask (Phi-3-small), None = dense."""
+    head_step, head0) block-sparse causal mask (Phi-3-small), None = dense.  ``keep_first`` > 0
+    (with a sliding ``window``): the first ``keep_first`` keys of the sequence stay visible after
+    they left the window (at their true positions)."""
     if not _gpu(q):
         r = ref.paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, window, k_scale, v_scale, softcap,
-                             sinks, alibi, row_lo, blocksparse)
+                             sinks, alibi, row_lo, blocksparse, keep_first)
         if out is not None:
             out.copy_(r)
             return out
         return r
     B, Hq, D = q.shape
     Hkv, P = k_cache.shape[1], k_cache.shape[2]
+    if q.dtype == torch.float32:   # fp32 models: the exact fp32 kernel (row b = sequence b at its last position)
+        _f32_only(softcap, sinks, alibi, row_lo, blocksparse)
+        return _paged_attention_f32(q, k_cache, v_cache, block_tables,
+                                    torch.arange(B, dtype=torch.int32, device=q.device), _i32(seq_lens) - 1, scale,
+                                    window, keep_first, out)
     if ws is None:
         ws = DecodeWorkspace(B, Hq, D, block_tables.shape[1] * P, device=q.device)
     out = torch.empty_like(q) if out is None else out
@@ -696,7 +814,28 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, ws: DecodeW
          out.stride(0), ws.part_o.data_ptr(), ws.part_ml.data_ptr(), B, Hq, Hkv, D, P, ws.part_size, ws.max_parts,
          float(scale), int(window), _i32(order).data_ptr() if order is not None else None, kv_format(k_cache),
          float(k_scale), float(v_scale), float(softcap), _sinks(sinks), _sinks(alibi),
-         _i32(row_lo).data_ptr() if row_lo is not None else None, blocksparse_pack(blocksparse), stream_ptr())
+         _i32(row_lo).data_ptr() if row_lo is not None else None, blocksparse_pack(blocksparse), int(keep_first),
+         stream_ptr())
+    return out
+
+
+def _f32_only(softcap, sinks, alibi, rows, blocksparse) -> None:
+    if softcap or sinks is not None or alibi is not None or rows is not None or blocksparse is not None:
+        raise NotImplementedError("fp32 attention: plain / windowed causal masks only")
+
+
+def _paged_attention_f32(q, k_cache, v_cache, block_tables, row_seq, row_pos, scale, window, keep_first, out):
+    """fp32 paged attention (``attention_f32.hip``): q [T, Hq, D] fp32, fp32 caches; row t belongs
+    to block-table row ``row_seq[t]`` and sits at absolute position ``row_pos[t]`` (< 0: padding)."""
+    T, Hq, D = q.shape
+    Hkv, P = k_cache.shape[1], k_cache.shape[2]
+    assert k_cache.dtype == v_cache.dtype == torch.float32 and q.stride(2) == 1 and q.stride(1) == D
+    out = torch.empty(T, Hq, D, dtype=q.dtype, device=q.device) if out is None else out
+    assert out.stride(2) == 1 and out.stride(1) == D
+    call("ome_paged_attention_f32", q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+         _i32(block_tables).data_ptr(), block_tables.stride(0), _i32(row_seq.contiguous()).data_ptr(),
+         _i32(row_pos.contiguous()).data_ptr(), out.data_ptr(), out.stride(0), T, Hq, Hkv, D, P, float(scale),
+         int(window), int(keep_first), stream_ptr())
     return out
 
 
@@ -1412,20 +1551,29 @@ def prefill_plan(q_lens: list[int], kv_lens: list[int], tile: int = 32, target: 
 def paged_prefill(q, k_cache, v_cache, block_tables, cu_q, kv_lens, items, scale, window: int = -1,
                   out=None, k_scale: float = 1.0, v_scale: float = 1.0, softcap: float = 0.0,
                   sinks: torch.Tensor | None = None, alibi: torch.Tensor | None = None,
-                  row_hi: torch.Tensor | None = None, blocksparse: tuple | None = None) -> torch.Tensor:
+                  row_hi: torch.Tensor | None = None, blocksparse: tuple | None = None,
+                  keep_first: int = 0) -> torch.Tensor:
     """q [Tq, Hq, D]; items int32 [n, 2] from :func:`prefill_work_items`.  ``softcap`` > 0:
     attention-logit soft-capping ``cap * tanh(score / cap)`` (Gemma-2); ``alibi``: fp32 [Hq]
     ALiBi slopes; ``row_hi``: int32 [Tq], per query row the last key position it may see
-    beyond the causal one (-1: causal) -- Gemma 3's bidirectional image blocks."""
+    beyond the causal one (-1: causal) -- Gemma 3's bidirectional image blocks.  ``keep_first``:
+    as in :func:`paged_decode`."""
     if not _gpu(q):
         r = ref.paged_prefill(q, k_cache, v_cache, block_tables, cu_q, kv_lens, scale, window, k_scale, v_scale,
-                              softcap, sinks, alibi, row_hi, blocksparse)
+                              softcap, sinks, alibi, row_hi, blocksparse, keep_first)
         if out is not None:
             out.copy_(r)
             return out
         return r
     Tq, Hq, D = q.shape
     Hkv, P = k_cache.shape[1], k_cache.shape[2]
+    if q.dtype == torch.float32:   # fp32 models: the exact fp32 kernel, one (sequence, position) per row
+        _f32_only(softcap, sinks, alibi, row_hi, blocksparse)
+        r = torch.arange(Tq, dtype=torch.int64, device=q.device)
+        seq = torch.bucketize(r, _i32(cu_q)[1:].long(), right=True).clamp_(max=cu_q.shape[0] - 2)
+        pos = _i32(kv_lens)[seq] - cu_q[seq + 1] + r
+        return _paged_attention_f32(q, k_cache, v_cache, block_tables, seq.to(torch.int32), pos.to(torch.int32),
+                                    scale, window, keep_first, out)
     out = torch.empty_like(q) if out is None else out
     rows = 32
     if isinstance(items, PrefillPlan):
@@ -1434,7 +1582,7 @@ def paged_prefill(q, k_cache, v_cache, block_tables, cu_q, kv_lens, items, scale
         if rows != 32 and not (rows == 64 and D == 128 and P == 16 and Hq == 4 * Hkv):
             raise ValueError(f"paged_prefill: {rows}-row items need the GQA-4 / D=128 kernel, got Hq={Hq} "
                              f"Hkv={Hkv} D={D} page={P} (build the plan with prefill_rows of this layer)")
-        if (plan.parts and D == 128 and P == 16 and Hq == 4 * Hkv and row_hi is None and
+        if (plan.parts and D == 128 and P == 16 and Hq == 4 * Hkv and row_hi is None and keep_first <= 0 and
                 os.environ.get("OME_PREFILL_ATTN", "2") == "2"):
             po = torch.empty(plan.parts * Hkv * 4 * 32 * 128, dtype=torch.float32, device=q.device)
             pml = torch.empty(plan.parts * Hkv * 4 * 32 * 2, dtype=torch.float32, device=q.device)
@@ -1443,14 +1591,15 @@ def paged_prefill(q, k_cache, v_cache, block_tables, cu_q, kv_lens, items, scale
                  _i32(kv_lens).data_ptr(), plan.split.data_ptr(), plan.split.shape[0], plan.comb.data_ptr(),
                  plan.comb.shape[0], int(plan.chunk), po.data_ptr(), pml.data_ptr(), out.data_ptr(), out.stride(0),
                  Hq, Hkv, float(scale), int(window), kv_format(k_cache), float(k_scale), float(v_scale),
-                 float(softcap), _sinks(sinks), _sinks(alibi), blocksparse_pack(blocksparse), stream_ptr())
+                 float(softcap), _sinks(sinks), _sinks(alibi), blocksparse_pack(blocksparse), int(keep_first),
+                 stream_ptr())
             return out
     call("ome_paged_prefill", q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
          _i32(block_tables).data_ptr(), block_tables.stride(0), _i32(cu_q).data_ptr(), _i32(kv_lens).data_ptr(),
          _i32(items).data_ptr(), items.shape[0], out.data_ptr(), out.stride(0), Hq, Hkv, D, P, float(scale),
          int(window), kv_format(k_cache), float(k_scale), float(v_scale), float(softcap), _sinks(sinks),
          _sinks(alibi), None if row_hi is None else _i32(row_hi).data_ptr(), rows, blocksparse_pack(blocksparse),
-         stream_ptr())
+         int(keep_first), stream_ptr())
     return out
 
 

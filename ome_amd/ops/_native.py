@@ -37,16 +37,23 @@ _SIGNATURES = {
         "ome_rope_qkv_cache": [vp, i64, vp, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp, vp, f32,
                                i32, f32, f32, vp],
         "ome_kv_cache_write": [vp, vp, i64, vp, vp, vp, i32, i32, i32, i32, i32, f32, f32, vp],
-        "ome_act_and_mul": [vp, vp, i64, i32, i32, vp],
+        "ome_act_and_mul": [vp, vp, i64, i32, i32, f32, vp],
+        "ome_embedding_f32": [vp, vp, vp, i32, i32, i32, f32, i32, vp],
+        "ome_residual_rmsnorm": [vp, i64, vp, i64, f32, vp, i64, f32, vp, vp, i64, i32, i32, f32, i32, vp],
+        "ome_wide_norm_rope_cache": [vp, i64, vp, i64, vp, i64, vp, vp, i32, i32, vp, vp, f32, vp, vp, vp, vp, i32,
+                                     i32, i32, i32, i32, i32, i32, i32, vp],
+        "ome_head_gate": [vp, vp, i64, vp, i32, i32, i32, i32, i32, i32, vp],
+        "ome_paged_attention_f32": [vp, i64, vp, vp, vp, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, f32, i32,
+                                    i32, vp],
         "ome_act": [vp, i64, i32, vp],
-        "ome_ssm_conv1d": [vp, i64, vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, vp],
+        "ome_ssm_conv1d": [vp, i64, vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, vp],
         "ome_dyn_conv1d": [vp, i64, vp, i64, i32, vp, i64, vp, vp, vp, vp, i32, i32, i32, vp],
         "ome_qk_norm_rope": [vp, i64, vp, vp, i32, i32, i32, f32, vp, i64, vp, vp],
         "ome_ssm_scan": [vp, i64, vp, i64, vp, vp, i64, vp, vp, vp, f32, vp, vp, i64, vp, vp, vp, i32, i32, i32,
-                         i32, i32, vp],
+                         i32, i32, i32, vp],
         "ome_gdn_scan": [vp, vp, vp, i64, vp, vp, i64, vp, vp, vp, vp, i64, vp, vp, vp, i32, i32, i32, i32, i32,
-                         i32, vp, vp],
-        "ome_gated_rmsnorm": [vp, i64, vp, i64, vp, vp, i64, i32, i32, i32, f32, i32, vp],
+                         i32, vp, i32, vp],
+        "ome_gated_rmsnorm": [vp, i64, vp, i64, vp, vp, i64, i32, i32, i32, f32, i32, i32, vp],
         "ome_layernorm": [vp, i64, vp, i64, vp, vp, vp, i64, i32, i32, f32, vp],
         "ome_embedding": [vp, vp, vp, i32, i32, i32, i32, vp],
         "ome_pool": [vp, vp, vp, i32, i32, i32, i32, vp],
@@ -62,11 +69,11 @@ _SIGNATURES = {
         "ome_moe_combine": [vp, vp, vp, i32, i32, i32, vp, f32, vp],
         "ome_moe_combine_add": [vp, vp, vp, i32, i32, i32, vp, vp, f32, vp],
         "ome_paged_decode": [vp, i64, vp, vp, vp, i32, vp, vp, i64, vp, vp, i32, i32, i32, i32, i32, i32, i32, f32,
-                             i32, vp, i32, f32, f32, f32, vp, vp, vp, i64, vp],
+                             i32, vp, i32, f32, f32, f32, vp, vp, vp, i64, i32, vp],
         "ome_paged_prefill": [vp, i64, vp, vp, vp, i32, vp, vp, vp, i32, vp, i64, i32, i32, i32, i32, f32, i32,
-                              i32, f32, f32, f32, vp, vp, vp, i32, i64, vp],
+                              i32, f32, f32, f32, vp, vp, vp, i32, i64, i32, vp],
         "ome_paged_prefill_split": [vp, i64, vp, vp, vp, i32, vp, vp, vp, i32, vp, i32, i32, vp, vp, vp, i64, i32,
-                                    i32, f32, i32, i32, f32, f32, f32, vp, vp, i64, vp],
+                                    i32, f32, i32, i32, f32, f32, f32, vp, vp, i64, i32, vp],
         "ome_varlen_attention": [vp, i64, vp, i64, vp, i64, vp, vp, vp, i32, vp, i64, i32, i32, i32, f32, i32, vp],
         "ome_skinny_gemm": [vp, i64, vp, vp, vp, i64, i32, i32, i32, i32, vp, vp, vp],
         "ome_w8a16_gemm": [vp, i64, vp, i64, vp, i32, vp, vp, i64, i32, i32, i32, i32, vp, vp, vp],

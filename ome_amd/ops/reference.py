@@ -66,7 +66,8 @@ def ssm_conv1d(x, w, bias, state, cu, slot, reset, out):
         o = torch.nn.functional.conv1d(seq.t()[None], w.float()[:, None, :], None if bias is None else bias.float(),
                                        groups=w.shape[0])[0].t()          # [L, C]
         out[r0:r1] = torch.nn.functional.silu(o).to(out.dtype)
-        st.copy_(seq[-(K - 1):].t().to(st.dtype))
+        if K > 1:
+            st.copy_(seq[-(K - 1):].t().to(st.dtype))
     return out
 
 
@@ -220,11 +221,11 @@ def kv_cache_write(k, v, k_cache, v_cache, slots, P, k_scale=1.0, v_scale=1.0) -
     v_cache[page, :, :, off] = to_cache(v, v_cache.dtype, v_scale)
 
 
-def act_and_mul(x: torch.Tensor, act: int = 0) -> torch.Tensor:
+def act_and_mul(x: torch.Tensor, act: int = 0, limit: float = 0.0) -> torch.Tensor:
     I = x.shape[-1] // 2
     g, u = x[..., :I].float(), x[..., I:].float()
     if act in (2, 3):  # clamped SwiGLU / GeGELU: GPT-OSS (limit 7), Phi-3-small (limit 20)
-        lim = 7.0 if act == 2 else 20.0
+        lim = float(limit) if limit and limit > 0 else (7.0 if act == 2 else 20.0)
         g = g.clamp(max=lim)
         u = u.clamp(-lim, lim)
         return ((u + 1) * g * torch.sigmoid(1.702 * g)).to(x.dtype)
@@ -238,6 +239,74 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, vocab_start: int = 0, voca
     local = torch.where(own, ids - vocab_start, torch.zeros_like(ids)).long()
     out = table[local]
     return out * own[:, None].to(out.dtype)
+
+
+def embedding_f32(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+    """fp32 rows ``table[ids] * scale`` (the start of an fp32 residual stream)."""
+    return table[ids.long()].float() * float(scale)
+
+
+def residual_rmsnorm(res, w, eps, x1=None, s1=1.0, x2=None, s2=1.0, out_dtype=None):
+    """fp32 residual stream: ``res += s1 * x1 + s2 * x2`` in place (either addend may be None),
+    then returns ``rmsnorm(res) * w`` in ``out_dtype``; everything in fp32 before the final cast."""
+    if x1 is not None:
+        res += float(s1) * x1.float() if x2 is None else float(s1) * x1.float() + float(s2) * x2.float()
+    rs = torch.rsqrt(res.pow(2).mean(-1, keepdim=True) + eps)
+    return (res * rs * w.float()).to(out_dtype or w.dtype)
+
+
+def wide_norm_rope_cache(q, k, v, positions, cos_sin, rot_dim, interleaved, qn_w, kn_w, eps, q_out, k_cache, v_cache,
+                         slots, Hq, Hkv, dim, vdim, P) -> None:
+    """Projection-wide q / k RMSNorm (one root mean square over ALL heads' channels of a row),
+    partial rotary on the first ``rot_dim`` dims of every head (``interleaved``: dim 2i pairs
+    with 2i+1; otherwise i with i + rot_dim/2), then q -> ``q_out`` [T, Hq, D] and k / v into the
+    paged cache (K [pages, Hkv, P, D], V [pages, Hkv, D, P]); head dims ``dim`` / ``vdim`` are
+    zero-padded to the cache's D."""
+    T = q.shape[0]
+    if T == 0:
+        return
+    D = k_cache.shape[3]
+    half = rot_dim // 2
+    cs = cos_sin[positions.long()].float()
+    cos, sin = cs[:, None, :half], cs[:, None, half:rot_dim]
+
+    def prep(x, w, H):
+        x = x.float()
+        if w is not None:
+            x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        x = x.view(T, H, dim).clone()
+        if rot_dim > 0:
+            if interleaved:
+                a, b = x[..., 0:rot_dim:2].clone(), x[..., 1:rot_dim:2].clone()
+                x[..., 0:rot_dim:2] = a * cos - b * sin
+                x[..., 1:rot_dim:2] = b * cos + a * sin
+            else:
+                a, b = x[..., :half].clone(), x[..., half:rot_dim].clone()
+                x[..., :half] = a * cos - b * sin
+                x[..., half:rot_dim] = b * cos + a * sin
+        return x
+
+    qf, kf = prep(q, qn_w, Hq), prep(k, kn_w, Hkv)
+    q_out.zero_()
+    q_out[:, :, :dim] = qf.to(q_out.dtype)
+    ok = slots >= 0
+    sl = slots[ok].long()
+    page, off = sl // P, sl % P
+    kp = torch.zeros(int(ok.sum()), Hkv, D, dtype=k_cache.dtype, device=k_cache.device)
+    kp[:, :, :dim] = kf[ok].to(k_cache.dtype)
+    vp = torch.zeros(int(ok.sum()), Hkv, D, dtype=v_cache.dtype, device=v_cache.device)
+    vp[:, :, :vdim] = v.reshape(T, Hkv, vdim)[ok].to(v_cache.dtype)
+    k_cache[page, :, off, :] = kp
+    v_cache[page, :, :, off] = vp
+
+
+def head_gate(o, g, vdim: int, kind: int = 0):
+    """``o`` [T, H, D] (attention output, head dim possibly padded) times ``sigmoid(g)`` (kind 0)
+    or ``silu(g)`` (kind 1), g [T, H * vdim] -> [T, H * vdim]."""
+    T, H, _ = o.shape
+    gf = g.float().view(T, H, vdim)
+    gate = torch.sigmoid(gf) if kind == 0 else torch.nn.functional.silu(gf)
+    return (o[:, :, :vdim].float() * gate).reshape(T, H * vdim).to(o.dtype)
 
 
 def gather_kv(k_cache, v_cache, block_table, n: int, kvh: int, P: int, k_scale=1.0, v_scale=1.0):
@@ -283,7 +352,8 @@ def blocksparse_visible(qpos: torch.Tensor, kpos: torch.Tensor, heads: torch.Ten
 
 
 def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, window=-1, k_scale=1.0,
-                 v_scale=1.0, softcap=0.0, sinks=None, alibi=None, row_lo=None, blocksparse=None) -> torch.Tensor:
+                 v_scale=1.0, softcap=0.0, sinks=None, alibi=None, row_lo=None, blocksparse=None,
+                 keep_first: int = 0) -> torch.Tensor:
     B, Hq, D = q.shape
     Hkv, P = k_cache.shape[1], k_cache.shape[2]
     G = Hq // Hkv
@@ -297,7 +367,14 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, window=-1, 
             lo = max(lo, int(row_lo[b]))
         for h in range(Hkv):
             k, v = gather_kv(k_cache, v_cache, block_tables[b], L, h, P, k_scale, v_scale)
-            k, v = k[lo:], v[lo:]
+            if keep_first > 0 and lo > keep_first:   # the kept first keys stay visible before the window
+                k, v = torch.cat([k[:keep_first], k[lo:]]), torch.cat([v[:keep_first], v[lo:]])
+                assert alibi is None and blocksparse is None
+            elif keep_first > 0:
+                k, v = k[0:], v[0:]
+                lo = 0
+            else:
+                k, v = k[lo:], v[lo:]
             qh = q[b, h * G:(h + 1) * G].float()
             s = _cap((qh @ k.T) * scale, softcap)
             if alibi is not None:  # slope * (key - query position)
@@ -314,7 +391,8 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, window=-1, 
 
 
 def paged_prefill(q, k_cache, v_cache, block_tables, cu_q, kv_lens, scale, window=-1, k_scale=1.0,
-                  v_scale=1.0, softcap=0.0, sinks=None, alibi=None, row_hi=None, blocksparse=None) -> torch.Tensor:
+                  v_scale=1.0, softcap=0.0, sinks=None, alibi=None, row_hi=None, blocksparse=None,
+                  keep_first: int = 0) -> torch.Tensor:
     Tq, Hq, D = q.shape
     Hkv, P = k_cache.shape[1], k_cache.shape[2]
     G = Hq // Hkv
@@ -329,7 +407,7 @@ def paged_prefill(q, k_cache, v_cache, block_tables, cu_q, kv_lens, scale, windo
         kpos = torch.arange(L, device=q.device)[None, :]
         qlim = qpos if row_hi is None else torch.maximum(qpos, row_hi[q0:q1].to(q.device).long()[:, None])
         mask = kpos <= qlim
-        mask &= kpos >= attn_lo(qpos, window)
+        mask &= (kpos >= attn_lo(qpos, window)) | (kpos < keep_first)
         for h in range(Hkv):
             k, v = gather_kv(k_cache, v_cache, block_tables[s], L, h, P, k_scale, v_scale)
             qh = q[q0:q1, h * G:(h + 1) * G].float().transpose(0, 1)  # [G, ql, D]
