@@ -77,14 +77,19 @@ class PagedKVCache:
         # ``num_kv_heads``: one count, or a {layer: heads} map (DeciLM / Nemotron-NAS: per-layer GQA)
         per = num_kv_heads if isinstance(num_kv_heads, dict) else None
         self.num_kv_heads = max(per.values()) if per else num_kv_heads
+        # ``head_dim``: one width, or a {layer: width} map (hybrids whose attention layers differ)
+        per_d = head_dim if isinstance(head_dim, dict) else None
+        head_dim = max(per_d.values()) if per_d else head_dim
         self.head_dim, self.dtype = head_dim, dtype
         self.v_dim = head_dim if v_dim is None else v_dim
         self.local_layers = list(range(num_layers)) if layers is None else list(layers)
         own = set(self.local_layers)
         hk = (lambda i: per[i]) if per else (lambda i: num_kv_heads)  # noqa: E731
-        self.k = [torch.zeros(num_pages, hk(i), page_size, head_dim, dtype=dtype, device=device)
+        hd = (lambda i: per_d[i]) if per_d else (lambda i: head_dim)  # noqa: E731
+        vd = (lambda i: per_d[i]) if per_d else (lambda i: self.v_dim)  # noqa: E731
+        self.k = [torch.zeros(num_pages, hk(i), page_size, hd(i), dtype=dtype, device=device)
                   if i in own else None for i in range(num_layers)]
-        self.v = [torch.zeros(num_pages, hk(i), self.v_dim, page_size, dtype=dtype, device=device)
+        self.v = [torch.zeros(num_pages, hk(i), vd(i), page_size, dtype=dtype, device=device)
                   if i in own else None for i in range(num_layers)]
         self.k_scale = [1.0] * num_layers
         self.v_scale = [1.0] * num_layers
@@ -105,9 +110,13 @@ class PagedKVCache:
     @staticmethod
     def bytes_per_page(num_layers: int, num_kv_heads: int, head_dim: int, page_size: int, dtype=torch.bfloat16,
                        v_dim: int | None = None) -> int:
+        esz = torch.tensor([], dtype=dtype).element_size()
+        if isinstance(head_dim, dict):   # per-layer widths (keys and values equally wide)
+            hk = num_kv_heads if isinstance(num_kv_heads, dict) else {i: num_kv_heads for i in head_dim}
+            return sum(hk[i] * 2 * d for i, d in head_dim.items()) * page_size * esz
         v = head_dim if v_dim is None else v_dim
         heads = sum(num_kv_heads.values()) if isinstance(num_kv_heads, dict) else num_layers * num_kv_heads
-        return heads * (head_dim + v) * page_size * torch.tensor([], dtype=dtype).element_size()
+        return heads * (head_dim + v) * page_size * esz
 
     def layer(self, i: int) -> tuple[torch.Tensor, torch.Tensor]:
         return self.k[i], self.v[i]

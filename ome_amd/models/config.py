@@ -40,6 +40,8 @@ def _standard_keys(c: dict[str, Any]) -> dict[str, Any]:
     the parser reads.  Existing standard keys win."""
     mt = c.get("model_type", "")
     a: dict[str, Any] = {}
+    if not mt and isinstance(c.get("layers"), list) and isinstance(c.get("architecture"), str):
+        return _layer_list_keys(c)
     if mt == "gptj":
         H, nh = c.get("n_embd", 4096), c.get("n_head", 16)
         a = dict(hidden_size=H, num_hidden_layers=c.get("n_layer"), num_attention_heads=nh,
@@ -128,6 +130,42 @@ def _standard_keys(c: dict[str, Any]) -> dict[str, Any]:
             out[k] = v
     return out
 
+
+
+def attn_tile_dim(d: int) -> int:
+    """Head width the attention / paged-cache kernels tile for ``d`` channels (zero-padded)."""
+    for t in (64, 128, 256):
+        if d <= t:
+            return t
+    raise ValueError(f"attention head width {d} exceeds the 256-wide kernel tile")
+
+
+def _layer_list_keys(c: dict[str, Any]) -> dict[str, Any]:
+    """Layer-list configs (``architecture: Zavilorn``): ``layers`` is a list of blocks, each with
+    its mixer ``type``, the mixer's own sizes and its feed-forward.  The standard keys describe the
+    envelope the runtime sizes its workspaces by (widest attention layer, fewest kv heads); the
+    model reads the per-layer entries from ``extra``."""
+    attn = [L["mixer"]["left"] for L in c["layers"] if L.get("type") == "parallel"]
+    ff = [L["mlp"]["ff"] for L in c["layers"] if L.get("mlp")]
+    D = max([attn_tile_dim(max(a["dim"], a["vdim"])) for a in attn] or [64])
+    out = dict(c)
+    out.update(architectures=[c["architecture"]], model_type=c["architecture"].lower(),
+               hidden_size=c["width"], vocab_size=c["vocab"], num_hidden_layers=len(c["layers"]),
+               rms_norm_eps=(c.get("norm") or {}).get("eps", 1e-6), tie_word_embeddings=True,
+               num_attention_heads=max([a["heads"] for a in attn] or [1]),
+               num_key_value_heads=min([a["kv_heads"] for a in attn] or [1]), head_dim=D,
+               intermediate_size=max(ff or [c["width"]]), rope_theta=(attn[0]["rot"]["base"] if attn else 10000.0),
+               partial_rotary_factor=(attn[0]["rot"]["dims"] / D if attn else 1.0),
+               max_position_embeddings=int(c.get("max_positions", 131072)), torch_dtype="bfloat16")
+    return out
+
+
+def plain_rope_table(base: float, rot_dim: int, max_pos: int, device=None) -> torch.Tensor:
+    """[max_pos, rot_dim] fp32 (cos | sin) for unscaled rotary frequencies base^(-2i/rot_dim)."""
+    inv = 1.0 / (float(base) ** (torch.arange(0, rot_dim, 2, dtype=torch.float64) / rot_dim))
+    fr = torch.outer(torch.arange(max_pos, dtype=torch.float64), inv)
+    cs = torch.cat([fr.cos(), fr.sin()], -1).float()
+    return cs.to(device) if device is not None else cs
 
 
 def _is_fp8_checkpoint(q: dict) -> bool:

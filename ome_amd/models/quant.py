@@ -208,7 +208,7 @@ def linear(x: torch.Tensor, w, bias: torch.Tensor | None = None, out: torch.Tens
             if copy:
                 return linear(x, w.bf16, bias)
         return ops.fp8_linear(x, w.q, w.scale, w.block, bias)
-    if x.dim() == 2 and x.shape[0] <= 256 and x.is_cuda:
+    if x.dim() == 2 and x.shape[0] <= 256 and x.is_cuda and x.dtype == torch.bfloat16:
         if x.shape[0] <= _GEMV_ROWS and ops.gemv_ok(x, w, bias):
             return ops.gemv(x, w, bias)
         plan = ops.decode_gemm_plan(x, w, bias)

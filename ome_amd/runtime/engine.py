@@ -95,6 +95,7 @@ class EngineArgs:
     decode_log_interval: int = 0           # --decode-log-interval: log decode throughput every N steps
                                            # (None = on for GPU engines)
     num_layers_override: int | None = None
+    keep_logits: bool = False              # replay / scoring: decode steps keep their rows' raw logits
     extra: dict = field(default_factory=dict)
 
     def model_config(self) -> ModelConfig:
@@ -151,7 +152,7 @@ class Engine:
                                   max_context=self.max_context, cuda_graph=args.cuda_graph,
                                   cuda_graph_max_bs=args.cuda_graph_max_bs, seed=args.seed,
                                   cuda_graph_bs=args.cuda_graph_bs,
-                                  kv_cache_dtype_name=args.kv_cache_dtype)
+                                  kv_cache_dtype_name=args.kv_cache_dtype, keep_logits=args.keep_logits)
         self.runner.pp_microbatches = args.pp_microbatches
         prefix = None
         m = self.runner.model
@@ -172,6 +173,7 @@ class Engine:
         self.served_model_name = args.served_model_name or (args.model_path or args.model or "model")
         self._lock = threading.Lock()
         self._inbox: list[Request] = []
+        self._replay: dict[str, Request] = {}   # live requests of a replayed trace, by id
         self._aborts: list[str] = []
         self._wake = threading.Event()
         self._stop = False
@@ -241,6 +243,40 @@ class Engine:
         pos, delta = mrope_positions(len(ids), spans, grids, m.merge)
         mm = MMInput(torch.cat(pvs, 0), grids, spans, pos, delta)
         return self.make_request(ids, params, mm=mm, **kw)
+
+    # ------------------------------------------------------------------ replay
+    def replay_step(self, entries: list[tuple[str, list[int], list[int]]], end: list[str] = ()):
+        """Teacher-forced step of a recorded trace: ``entries`` = (request id, its next tokens,
+        indices among them whose logits are wanted).  The entries run as one batch through the
+        scheduler's admission / paging (:meth:`Scheduler.forced_batch`) and the model runner's
+        step (HIP-graph decode when every entry is a single token, the eager mixed step
+        otherwise); requests named in ``end`` are finished afterwards (pages and state slot go
+        back to the pools).  Returns the wanted logits, fp32 [rows, vocab] on the host, in entry
+        order (None when nothing was wanted)."""
+        if not self.runner.keep_logits:
+            raise RuntimeError("replay needs EngineArgs(keep_logits=True)")
+        live = self._replay
+        parts = []
+        for rid, tokens, want in entries:
+            r = live.get(rid)
+            if r is None:
+                r = live[rid] = Request(prompt_ids=[], params=SamplingParams(max_new_tokens=0), rid=rid)
+            r.prompt_ids.extend(int(t) for t in tokens)
+            parts.append((r, len(tokens), want))
+        out = None
+        if parts:
+            batch = self.scheduler.forced_batch(parts)
+            handle = self.runner.launch(batch, None)
+            self.scheduler.launch_commit(batch)
+            handle.result()
+            self.step_count += 1
+            if handle.logits is not None:
+                out = handle.logits.float().cpu()
+        for rid in end:
+            r = live.pop(rid, None)
+            if r is not None:
+                self.scheduler.finish(r, "stop")
+        return out
 
     def add_request(self, req: Request) -> Request:
         with self._lock:

@@ -110,10 +110,13 @@ class StepHandle:
     """An enqueued step: device outputs (for the next step's pending-token gather) plus the
     pinned host copies that ``result()`` waits for."""
 
-    __slots__ = ("ids_dev", "n", "host_ids", "host_lp", "event")
+    __slots__ = ("ids_dev", "n", "host_ids", "host_lp", "event", "logits")
 
-    def __init__(self, ids_dev, n, host_ids, host_lp, event):
+    def __init__(self, ids_dev, n, host_ids, host_lp, event, logits=None):
         self.ids_dev, self.n, self.host_ids, self.host_lp, self.event = ids_dev, n, host_ids, host_lp, event
+        # fp32 [rows, vocab] device tensor: the logits of the rows the batch's chunks asked for
+        # (``ScheduledChunk.want``), in chunk order; None when no chunk asked
+        self.logits = logits
 
     def result(self) -> tuple[list[int], list[float]]:
         if self.event is not None:
@@ -145,8 +148,10 @@ class ModelRunner:
                  model_path: str | None = None, load_format: str = "auto", page_size: int = 16,
                  mem_fraction_static: float = 0.9, max_total_tokens: int | None = None, max_running: int = 256,
                  max_context: int = 8192, cuda_graph: bool = True, cuda_graph_max_bs: int | None = None,
-                 seed: int = 0, kv_cache_dtype_name: str = "auto", cuda_graph_bs: list | None = None):
+                 seed: int = 0, kv_cache_dtype_name: str = "auto", cuda_graph_bs: list | None = None,
+                 keep_logits: bool = False):
         self.cfg = cfg
+        self.keep_logits = bool(keep_logits)
         self.device = torch.device(device)
         self.dtype = dtype
         self.P = page_size
@@ -184,6 +189,8 @@ class ModelRunner:
         n_local = len(self.model.layers if kv_layers is None else kv_layers)
         if getattr(self.model, "kv_heads_per_layer", None):   # per-layer GQA (DeciLM): {layer: local heads}
             kv_heads = dict(self.model.kv_heads_per_layer)
+        if getattr(self.model, "kv_dims_per_layer", None):    # per-layer head widths: {layer: D}
+            k_dim, v_dim = dict(self.model.kv_dims_per_layer), None
         kv_dtype = kv_cache_dtype(kv_cache_dtype_name, dtype)
         if kv_dtype != dtype and getattr(self.model, "kv_layout", None) is not None:
             # MLA's latent cache (mla.hip) keeps the model dtype
@@ -257,6 +264,8 @@ class ModelRunner:
         self.counts = torch.zeros(max_running + 1, cfg.vocab_size, dtype=torch.int32, device=self.device)
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.graph_pool = None
+        self._dec_logits: dict = {}
+        self._want_logits = None
         # pipeline stages capture their decode step when every hand-off is an IPC peer kernel
         # (pstate.pp_graph_ok: one node); across nodes they run eagerly over RCCL p2p.  DP
         # attention replays graphs only with the low-latency EP exchange (cuda_graph=None: "if possible")
@@ -394,6 +403,9 @@ class ModelRunner:
             hidden = self.model.forward(d.view("ids", bs), meta, self.kv)
         if hidden is not None:   # (an earlier pipeline stage returns None: it samples nothing)
             logits = self.model.compute_logits(hidden)
+            if self.keep_logits:   # raw logits of every row, before penalties (graph-pool memory when
+                # captured: the reference keeps it from being reused by later captures)
+                self._dec_logits[(m, bs)] = logits.float() if logits.dtype != torch.float32 else logits.clone()
             pen = (d.view("rep", bs), d.view("freq", bs), d.view("pres", bs))
             ops.apply_penalties(logits, self.counts, d.view("req_idx", bs), *pen)
             ops.sample(logits, d.view("temp", bs), d.view("top_k", bs), d.view("top_p", bs), d.view("min_p", bs),
@@ -608,7 +620,9 @@ class ModelRunner:
             self._decode_forward(bs)
         if self.pp:
             pstate.pp_broadcast_tokens(self.out_ids[:B], self.out_lp[:B])
-        return self._finish_launch(self.out_ids, self.out_lp, B)
+        h = self._finish_launch(self.out_ids, self.out_lp, B)
+        h.logits = self._wanted_decode_logits(batch.chunks, bs)
+        return h
 
     def _fill_decode(self, d: "_DecodeBuffers", chunks, bs: int, prev: "StepHandle | None") -> None:
         """Host-side fields of a decode (micro-)batch -> ``d``'s pinned image -> one H2D copy."""
@@ -670,6 +684,18 @@ class ModelRunner:
             ops.fill_pending(d.view("ids", bs), d.view("src", bs), prev.ids_dev)
 
     pp_microbatches = 0   # pipeline parallel: micro-batches per step (0 = one per stage)
+    # replay / scoring mode (set before the decode graphs are captured): decode steps keep the raw
+    # logits of their rows so chunks can ask for them (``ScheduledChunk.want``)
+    keep_logits = False
+
+    def _wanted_decode_logits(self, chunks, bs: int, m: int = 0):
+        rows = [i for i, c in enumerate(chunks) if getattr(c, "want", None)]
+        if not rows:
+            return None
+        if not self.keep_logits:
+            raise RuntimeError("decode steps return logits only in keep_logits mode")
+        idx = torch.tensor(rows, dtype=torch.long, device=self.device)
+        return self._dec_logits[(m, bs)].index_select(0, idx)
 
     def _launch_eager(self, batch: StepBatch, prev: "StepHandle | None") -> "StepHandle":
         """Eager step for prefill / mixed batches (and every step of a pipeline-parallel engine).
@@ -691,7 +717,9 @@ class ModelRunner:
             out_ids, out_lp = self._eager_forward(chunks, prev, batch.mode)
         if self.pp:
             pstate.pp_broadcast_tokens(out_ids, out_lp)
-        return self._finish_launch(out_ids, out_lp, len(chunks))
+        h = self._finish_launch(out_ids, out_lp, len(chunks))
+        h.logits, self._want_logits = self._want_logits, None
+        return h
 
     def _eager_forward(self, chunks, prev: "StepHandle | None", mode: str) -> tuple[torch.Tensor, torch.Tensor]:
         """One eager forward over ``chunks``: (sampled ids int32, log-probs fp32) in chunk order;
@@ -738,6 +766,8 @@ class ModelRunner:
         # its kv heads per layer; the plan is shared by all layers)
         hkvs = set(getattr(self.model, "kv_heads_per_layer", {}).values()) | {tp_.hkv}
         rows = ops.prefill_rows(tp_.hq, tp_.hkv, self.cfg.head_dim, P) if len(hkvs) == 1 else 32
+        if hasattr(self.model, "prefill_item_rows"):   # layers of different attention shapes
+            rows = self.model.prefill_item_rows(P)
         items, split, comb, chunk, parts = ops.prefill_plan(q_lens, kv_lens, tile=rows, kv_heads=tp_.hkv) if q_lens \
             else ([], [], [], 0, 0)
         T, S, n_it, nd, B = len(ids), len(q_lens), len(items), len(dec_lens), len(chunks)
@@ -825,6 +855,11 @@ class ModelRunner:
         if hidden is None:  # an earlier pipeline stage: tokens arrive from the last stage
             return (torch.empty(len(chunks), dtype=torch.int32, device=self.device),
                     torch.empty(len(chunks), dtype=torch.float32, device=self.device))
+        want = [last_row[i] - c.length + 1 + w for i, c in enumerate(chunks) for w in (getattr(c, "want", None) or ())]
+        if want:   # scoring: logits of arbitrary rows of the chunks (prompt positions), chunk order
+            wl = self.model.compute_logits(hidden.index_select(0, torch.tensor(want, dtype=torch.long,
+                                                                               device=self.device)))
+            self._want_logits = wl.float()
         logits = self.model.compute_logits(hidden.index_select(0, t_rows))
         pen = None
         if any(c.req.params.has_penalties for c in chunks):

@@ -29,6 +29,7 @@ class ScheduledChunk:
     length: int     # tokens computed this step
     sample: bool    # last row produces a new token
     out_index: int = -1   # index in req.output_ids the sampled token lands at (set at launch)
+    want: list | None = None   # rows of this chunk (0-based) whose logits the step returns (scoring)
 
 
 @dataclass
@@ -333,6 +334,36 @@ class Scheduler:
         # a later request's page growth may have preempted one already picked (LIFO victim)
         chunks = [c for c in chunks if c.req.state == ReqState.RUNNING and len(c.req.pages) * self.P >= c.req.seq_len]
         return StepBatch("decode", chunks) if chunks else None
+
+    # ------------------------------------------------------------------ replay
+    def forced_batch(self, parts: list[tuple[Request, int, list | None]]) -> StepBatch:
+        """A step dictated from outside (trace replay / scoring): ``parts`` = (request, number of
+        its next tokens to run, rows whose logits are wanted).  New requests are admitted (state
+        slot + pages), known ones continue from their cache watermark; nothing is sampled.  All
+        parts form ONE batch -- chunks of several tokens beside single-token rows -- exactly as a
+        scheduled mixed step would.  Raises when slots or pages run out (the caller sized them)."""
+        chunks = []
+        for r, n, want in parts:
+            if n <= 0 or r.num_cached + n > r.seq_len:
+                raise ValueError(f"{r.rid}: cannot run {n} tokens from position {r.num_cached} of {r.seq_len}")
+            if r.num_cached + n > self.max_context:
+                raise ValueError(f"{r.rid}: {r.num_cached + n} tokens exceed the context length {self.max_context}")
+            if r.state != ReqState.RUNNING:
+                if r in self.waiting:
+                    self.waiting.remove(r)
+                if r.req_slot < 0:
+                    slot = self.slots.alloc()
+                    if slot is None:
+                        raise RuntimeError("no free request slot")
+                    r.req_slot = slot
+                r.state = ReqState.RUNNING
+                self.running.append(r)
+            if not self._grow(r, r.num_cached + n):
+                raise RuntimeError(f"{r.rid}: out of KV pages ({self.pages.num_free} free)")
+            chunks.append(ScheduledChunk(r, r.num_cached, n, False, want=list(want) if want else None))
+        # a decode step continues every row's recurrent state: a request's very first token (even
+        # alone) is a prefill chunk, as in scheduled serving, so its state slot starts from zero
+        return StepBatch("decode" if all(c.length == 1 and c.start > 0 for c in chunks) else "prefill", chunks)
 
     # ------------------------------------------------------------------ post-step
     def launch_commit(self, batch: StepBatch) -> None:
