@@ -258,6 +258,8 @@ class Engine:
         live = self._replay
         parts = []
         for rid, tokens, want in entries:
+            if not tokens:
+                continue
             r = live.get(rid)
             if r is None:
                 r = live[rid] = Request(prompt_ids=[], params=SamplingParams(max_new_tokens=0), rid=rid)
