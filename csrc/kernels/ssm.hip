@@ -185,8 +185,10 @@ template <typename T>
 __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const T* __restrict__ y, int64_t y_stride,
                                                             const T* __restrict__ z, int64_t z_stride,
                                                             const T* __restrict__ w, T* __restrict__ out,
-                                                            int64_t out_stride, int group, float eps, int norm_first) {
+                                                            int64_t out_stride, int group, float eps, int mode) {
   __shared__ float red[4];
+  const int norm_first = mode & 1;
+  const bool exact = (mode & 2) != 0;
   const int row = blockIdx.y, g0 = blockIdx.x * group;
   const T* yr = y + (int64_t)row * y_stride + g0;
   const T* zr = z + (int64_t)row * z_stride + g0;
@@ -199,7 +201,10 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const T* __restrict_
   const float rs = 1.f / sqrtf(tot / (float)group + eps);
   T* orow = out + (int64_t)row * out_stride + g0;
   for (int i = threadIdx.x; i < group; i += 256) {
-    if (norm_first) {   // Qwen3-Next: w (per group channel) * norm(y), then * silu(z)
+    if (exact) {        // one rounding, at the store (models that keep their norms in fp32)
+      const float zs = silu_f((float)zr[i]);
+      orow[i] = (T)(norm_first ? (float)yr[i] * rs * (float)w[i] * zs : (float)yr[i] * zs * rs * (float)w[g0 + i]);
+    } else if (norm_first) {   // Qwen3-Next: w (per group channel) * norm(y), then * silu(z)
       const float t = (float)(T)((float)(T)((float)yr[i] * rs) * (float)w[i]);
       orow[i] = (T)(t * silu_f((float)zr[i]));
     } else {
@@ -418,7 +423,7 @@ OME_API int ome_ssm_scan(const void* x, int64_t x_stride, const void* dt, int64_
 
 OME_API int ome_gated_rmsnorm(const void* y, int64_t y_stride, const void* z, int64_t z_stride, const void* w,
                               void* out, int64_t out_stride, int rows, int I, int group, float eps,
-                              int norm_first, int f32, hipStream_t stream) {
+                              int norm_first, int f32, hipStream_t stream) {   // norm_first | 2: no intermediate rounding
   if (rows <= 0) return 0;
   if (group <= 0 || I % group != 0) return -2;
   dim3 grid(I / group, rows);

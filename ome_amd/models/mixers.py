@@ -167,7 +167,7 @@ class GatedDeltaMixer(_Block):
         c = ops.ssm_conv1d(p[:, :cd], self.conv_w, None, self.conv_state, cu, slot, reset)
         o = ops.gdn_scan(c[:, :kd], c[:, kd:2 * kd], c[:, 2 * kd:], p[:, cd + vd + Hv:], p[:, cd + vd:cd + vd + Hv],
                          self.A_log, self.dt_bias, self.rec_state, cu, slot, reset, Hv, self.Hk)
-        o = ops.gated_rmsnorm(o, p[:, cd:cd + vd], self.gnorm, self.dv, self.eps, norm_first=True)
+        o = ops.gated_rmsnorm(o, p[:, cd:cd + vd], self.gnorm, self.dv, self.eps, norm_first=True, exact=True)
         return linear(o, self.w_o)
 
 
@@ -218,7 +218,7 @@ class Mamba2Mixer(_Block):
         c = ops.ssm_conv1d(p[:, I:I + cd], self.conv_w, self.conv_b, self.conv_state, cu, slot, reset)
         y = ops.ssm_scan(c[:, :I], p[:, I + cd:], c[:, I:I + GN], c[:, I + GN:], self.A, self.Dp, self.dt_bias, 0.0,
                          self.ssm_state, cu, slot, reset, self.H, self.P, self.N, self.G)
-        y = ops.gated_rmsnorm(y, p[:, :I], self.gnorm, self.norm_group, self.eps)
+        y = ops.gated_rmsnorm(y, p[:, :I], self.gnorm, self.norm_group, self.eps, exact=True)
         return linear(y, self.w_o)
 
 

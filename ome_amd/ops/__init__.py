@@ -200,15 +200,17 @@ def gdn_scan(q, k, v, a, b, A_log, dt_bias, state, cu, slot, reset, Hv: int, Hk:
 
 
 def gated_rmsnorm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, group: int, eps: float,
-                  norm_first: bool = False) -> torch.Tensor:
+                  norm_first: bool = False, exact: bool = False) -> torch.Tensor:
     """w * groupRMSNorm(y * silu(z)) (Mamba-2 output norm, groups of ``group`` channels);
-    ``norm_first``: w[:group] * groupRMSNorm(y) * silu(z) (Qwen3-Next, ``w`` shared by the groups)."""
+    ``norm_first``: w[:group] * groupRMSNorm(y) * silu(z) (Qwen3-Next, ``w`` shared by the groups).
+    ``exact``: the whole expression in fp32 with one rounding at the store (default: the
+    normalised value is rounded to the model dtype before the scale, as HF's modules do)."""
     if not _gpu(y):
-        return ref.gated_rmsnorm(y, z, w, group, eps, norm_first)
+        return ref.gated_rmsnorm(y, z, w, group, eps, norm_first, exact)
     T, I = y.shape
     out = torch.empty(T, I, dtype=y.dtype, device=y.device)
     call("ome_gated_rmsnorm", y.data_ptr(), y.stride(0), z.data_ptr(), z.stride(0), w.data_ptr(), out.data_ptr(),
-         out.stride(0), T, I, group, float(eps), int(norm_first), _f32(y, z, w), stream_ptr())
+         out.stride(0), T, I, group, float(eps), int(norm_first) | (2 if exact else 0), _f32(y, z, w), stream_ptr())
     return out
 
 

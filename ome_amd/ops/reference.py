@@ -154,8 +154,16 @@ def gdn_scan(q, k, v, a, b, A_log, dt_bias, state, cu, slot, reset, Hv, Hk, out)
     return out
 
 
-def gated_rmsnorm(y, z, w, group, eps, norm_first=False):
+def gated_rmsnorm(y, z, w, group, eps, norm_first=False, exact=False):
     T, I = y.shape
+    if exact:   # fp32 throughout, one rounding at the end
+        zs = torch.nn.functional.silu(z.float())
+        v = y.float() if norm_first else y.float() * zs
+        g = v.view(T, I // group, group)
+        g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
+        if norm_first:
+            return (g * w.float()[:group] * zs.view(T, I // group, group)).view(T, I).to(y.dtype)
+        return (g.view(T, I) * w.float()).to(y.dtype)
     if norm_first:
         g = y.float().view(T, I // group, group)
         g = (g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)).to(y.dtype)

@@ -318,9 +318,13 @@ def test_float32_ops_match_reference():
     assert tight(g0, g_r)
     yy, zz, ww = f(9, 48), f(9, 48), torch.rand(48, device=DEV) + 0.5
     for nf in (False, True):
-        wv = ww[:12] if nf else ww
-        assert tight(ops.gated_rmsnorm(yy, zz, wv, 12, 1e-6, norm_first=nf), ref.gated_rmsnorm(c(yy), c(zz), c(wv), 12,
-                                                                                               1e-6, nf))
+        for ex in (False, True):
+            wv = ww[:12].contiguous() if nf else ww
+            assert tight(ops.gated_rmsnorm(yy, zz, wv, 12, 1e-6, norm_first=nf, exact=ex),
+                         ref.gated_rmsnorm(c(yy), c(zz), c(wv), 12, 1e-6, nf, ex))
+            yb, zb, wb = yy.to(BF), zz.to(BF), wv.to(BF)
+            assert _close(ops.gated_rmsnorm(yb, zb, wb, 12, 1e-6, norm_first=nf, exact=ex),
+                          ref.gated_rmsnorm(c(yb), c(zb), c(wb), 12, 1e-6, nf, ex), 1e-2)
 
 
 @pytest.mark.parametrize("window,keep", [(-1, 0), (9, 3), (40, 0), (2000, 5)])
