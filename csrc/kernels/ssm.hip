@@ -1,7 +1,7 @@
 // Mamba-2 (selective state space) kernels for hybrid models (NemotronH; reference catalog
 // ``NemotronHForCausalLM`` runtimes), CDNA4 / gfx950.
 //
-//   ome_ssm_conv1d       : causal depthwise conv (kernel K <= 8) + SiLU over a varlen batch of
+//   ome_ssm_conv1d       : causal depthwise conv (K <= 32 taps) + SiLU over a varlen batch of
 //                          sequences, continuing from / updating each sequence's conv state
 //   ome_dyn_conv1d       : the same with per-row (input-generated) taps (Jet-Nemotron JetBlock)
 //   ome_ssm_scan         : the selective scan  h <- exp(dt*A) h + dt * B x,  y = C.h + D x
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const T* __restrict_
 }
 
 
-// Any tap count 1 <= K <= 16 (the templated kernels cover 2..6): same arguments, runtime loops.
+// Any tap count 1 <= K <= 32 (the templated kernels cover 2..6): same arguments, runtime loops.
 template <typename T>
 __global__ __launch_bounds__(256) void ssm_conv1d_any_kernel(const T* __restrict__ x, int64_t x_stride,
                                                              const T* __restrict__ w, const T* __restrict__ bias,
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256) void ssm_conv1d_any_kernel(const T* __restrict
   const int r0 = cu[s], r1 = cu[s + 1];
   if (r1 <= r0) return;
   T* st = state + ((int64_t)slot[s] * C + c) * (K - 1);
-  float win[15], wt[16];
+  float win[31], wt[32];
   const bool fresh = reset[s] != 0;
   for (int j = 0; j < K - 1; ++j) win[j] = fresh ? 0.f : (float)st[j];
   for (int j = 0; j < K; ++j) wt[j] = (float)w[(int64_t)c * K + j];
@@ -302,7 +302,7 @@ OME_API int ome_ssm_conv1d(const void* x, int64_t x_stride, const void* w, const
   if (S <= 0 || C <= 0) return 0;
   dim3 grid((C + 255) / 256, S);
   if (f32) {   // fp32 models: inputs, taps, outputs and the tail state are float
-    if (K < 1 || K > 16) return -2;
+    if (K < 1 || K > 32) return -2;
     ssm_conv1d_any_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, (const float*)w,
                                                            (const float*)bias, (float*)out, out_stride,
                                                            (float*)state, cu, slot, reset, C, K);
@@ -321,7 +321,7 @@ OME_API int ome_ssm_conv1d(const void* x, int64_t x_stride, const void* w, const
     CONV_CASE(5)
     CONV_CASE(6)
     default:
-      if (K < 1 || K > 16) return -2;
+      if (K < 1 || K > 32) return -2;
       ssm_conv1d_any_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)x, x_stride, (const bf16*)w, (const bf16*)bias,
                                                       (bf16*)out, out_stride, (bf16*)state, cu, slot, reset, C, K);
       break;

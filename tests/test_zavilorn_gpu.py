@@ -148,7 +148,7 @@ def test_gdn_scan_any_shape(dk, dv, Hk, Hv, pad):
     assert torch.equal(st_k[1].cpu(), st0[1].cpu())
 
 
-@pytest.mark.parametrize("K", [1, 3, 7, 9])
+@pytest.mark.parametrize("K", [1, 3, 7, 9, 20])
 def test_conv_any_taps(K):
     torch.manual_seed(5)
     C, lens = 37, [4, 1, 19]
