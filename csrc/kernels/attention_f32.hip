@@ -8,6 +8,8 @@
 // attention (window < -1), kept first keys.  They are visited in chunks of CH keys: one thread per
 // key forms q.k, the block reduces max and sum (online softmax across chunks), then one thread per
 // output dim accumulates p.V.  Built for exactness at test sizes, not for speed.
+// sinks (optional, fp32 [Hq]): a per-head logit that joins the softmax denominator once, unscaled,
+// with no key and no value (exp(sink) is added to the sum of the weights).
 #include "common.h"
 
 namespace {
@@ -28,7 +30,7 @@ __global__ __launch_bounds__(256) void paged_attention_f32_kernel(
     const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k_cache,
     const float* __restrict__ v_cache, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ row_seq, const int* __restrict__ row_pos, float* __restrict__ out, int64_t out_stride,
-    int Hq, int Hkv, int D, int P, float scale, int window, int keep) {
+    int Hq, int Hkv, int D, int P, float scale, int window, int keep, const float* __restrict__ sinks) {
   __shared__ float qs[256];
   __shared__ float sc[CH];
   __shared__ float red[4];
@@ -81,6 +83,11 @@ __global__ __launch_bounds__(256) void paged_attention_f32_kernel(
     }
     __syncthreads();
   }
+  if (sinks != nullptr) {
+    const float sk = sinks[h], m_new = fmaxf(m, sk), alpha = expf(m - m_new);
+    l = l * alpha + expf(sk - m_new);
+    acc *= alpha;
+  }
   if (tid < D) orow[tid] = acc / l;
 }
 
@@ -89,12 +96,13 @@ __global__ __launch_bounds__(256) void paged_attention_f32_kernel(
 OME_API int ome_paged_attention_f32(const float* q, int64_t q_stride, const float* k_cache, const float* v_cache,
                                     const int* block_tables, int bt_stride, const int* row_seq, const int* row_pos,
                                     float* out, int64_t out_stride, int T, int Hq, int Hkv, int D, int P, float scale,
-                                    int window, int keep_first, hipStream_t stream) {
+                                    int window, int keep_first, const float* sinks, hipStream_t stream) {
   if (T <= 0) return 0;
   if (D <= 0 || D > 256 || P <= 0 || Hkv <= 0 || Hq % Hkv != 0) return -2;
   paged_attention_f32_kernel<<<dim3(T, Hq), 256, 0, stream>>>(q, q_stride, k_cache, v_cache, block_tables, bt_stride,
                                                               row_seq, row_pos, out, out_stride, Hq, Hkv, D, P, scale,
-                                                              window, window > 0 && keep_first > 0 ? keep_first : 0);
+                                                              window, window > 0 && keep_first > 0 ? keep_first : 0,
+                                                              sinks);
   OME_CHECK_LAUNCH();
   return 0;
 }

@@ -311,3 +311,59 @@ OME_API int ome_head_gate(const void* o, const void* g, int64_t g_stride, void* 
   OME_CHECK_LAUNCH();
   return 0;
 }
+
+// Per-token gated side input: out[t, j] = gelu_tanh(g[t, j]) * table[ids[t], col0 + j], j < n
+// (g: a projection's output; table: a second embedding table whose row holds every layer's part,
+// this layer's starting at column col0).  Product in fp32, one rounding.
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_gather_mul_kernel(const T* __restrict__ g, int64_t g_stride,
+                                                              const int* __restrict__ ids,
+                                                              const T* __restrict__ table, int64_t t_stride, int V,
+                                                              int col0, T* __restrict__ out, int n, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / n;
+  const int j = (int)(i - t * n);
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+  out[i] = (T)(gelu_tanh((float)g[t * g_stride + j]) * (float)table[(int64_t)id * t_stride + col0 + j]);
+}
+
+OME_API int ome_gelu_gather_mul(const void* g, int64_t g_stride, const int* ids, const void* table, int64_t t_stride,
+                                int V, int col0, void* out, int T, int n, int f32, hipStream_t stream) {
+  if (T <= 0 || n <= 0) return 0;
+  const int64_t total = (int64_t)T * n;
+  const int blocks = (int)((total + 255) / 256);
+  if (f32)
+    gelu_gather_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)g, g_stride, ids, (const float*)table,
+                                                              t_stride, V, col0, (float*)out, n, total);
+  else
+    gelu_gather_mul_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)g, g_stride, ids, (const bf16*)table,
+                                                             t_stride, V, col0, (bf16*)out, n, total);
+  OME_CHECK_LAUNCH();
+  return 0;
+}
+
+// Rows of a mixture of experts whose router weight scales the expert's INPUT: out[t * k + j, :] =
+// w[t, j] * x[t, :] (fp32 product, one rounding) -- the expanded, pre-scaled rows the grouped GEMM
+// then sorts by expert.
+template <typename T>
+__global__ __launch_bounds__(256) void scale_rows_kernel(const T* __restrict__ x, int64_t x_stride,
+                                                         const float* __restrict__ w, int k, T* __restrict__ out,
+                                                         int H) {
+  const int64_t r = blockIdx.x;            // expanded row t * k + j
+  const float wv = w[r];
+  const T* xr = x + (r / k) * x_stride;
+  for (int i = threadIdx.x; i < H; i += 256) out[r * H + i] = (T)(wv * (float)xr[i]);
+}
+
+OME_API int ome_scale_rows(const void* x, int64_t x_stride, const float* w, int k, void* out, int T, int H, int f32,
+                           hipStream_t stream) {
+  if (T <= 0 || k <= 0) return 0;
+  if (f32)
+    scale_rows_kernel<float><<<T * k, 256, 0, stream>>>((const float*)x, x_stride, w, k, (float*)out, H);
+  else
+    scale_rows_kernel<bf16><<<T * k, 256, 0, stream>>>((const bf16*)x, x_stride, w, k, (bf16*)out, H);
+  OME_CHECK_LAUNCH();
+  return 0;
+}

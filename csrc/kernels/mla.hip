@@ -508,3 +508,85 @@ OME_API int ome_mla_prep(const void* a, int64_t lda, int qlr, int lat, int rope,
                                          qf_tok, qf_head);
   return (int)hipGetLastError();
 }
+
+// ------------------------------------------------------------------------------------------
+// Latent-attention glue for the generic paged attention kernels (any latent width / rotary width,
+// bf16 or fp32): the absorbed form is multi-query attention with ONE shared head whose key is
+// [RMSNorm(c) * w | rotated k_pe] and whose value is the latent RMSNorm(c) * w itself.  From the
+// fused down-projection output a [T, qlr + lat + rope] this writes, per token,
+//   K cache row   [page, 0, off, 0 : lat + rope]  (row-major keys, head width D >= lat + rope)
+//   V cache column [page, 0, 0 : lat, off]        (the value layout of the attention kernels)
+// (the tails up to D are never written: the caches start as zeros) and, for every head, the rotated
+// q_pe into qf[t, h, lat : lat + rope] with zeros up to D.  Rotary pairs are (j, j + rope/2), angles
+// from the fp32 table row of the token's position (cos | sin, any frequency scaling baked in).
+// k_cache == nullptr: a layer that reads another layer's cache only rotates its queries.
+// Padding rows (slot < 0) write slot 0 of the scratch page.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prep_kernel(
+    const T* __restrict__ a, int64_t lda, int qlr, int lat, int rope, const T* __restrict__ w, float eps,
+    const int* __restrict__ pos, const float* __restrict__ cs, const int* __restrict__ slots,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int D, int P, const T* __restrict__ q, int64_t q_tok,
+    int64_t q_head, int nope, int H, T* __restrict__ qf, int64_t qf_tok, int64_t qf_head) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int half = rope >> 1;
+  const float* c = cs + (int64_t)pos[t] * rope;
+  if (k_cache != nullptr) {
+    const T* ar = a + (int64_t)t * lda + qlr;
+    int slot = slots[t];
+    slot = slot < 0 ? 0 : slot;
+    T* krow = k_cache + (int64_t)slot * D;
+    T* vcol = v_cache + (int64_t)(slot / P) * D * P + slot % P;
+    float ss = 0.f;
+    for (int i = tid; i < lat; i += 256) {
+      const float v = (float)ar[i];
+      ss += v * v;
+    }
+    ss = block_sum<256>(ss, red);
+    const float rs = 1.f / sqrtf(ss / (float)lat + eps);
+    for (int i = tid; i < lat; i += 256) {
+      const T v = (T)((float)ar[i] * rs * (float)w[i]);
+      krow[i] = v;
+      vcol[(int64_t)i * P] = v;
+    }
+    for (int j = tid; j < half; j += 256) {
+      const float x1 = (float)ar[lat + j], x2 = (float)ar[lat + half + j];
+      const float co = c[j], si = c[half + j];
+      krow[lat + j] = (T)(x1 * co - x2 * si);
+      krow[lat + half + j] = (T)(x2 * co + x1 * si);
+    }
+  }
+  const int tail = D - lat - rope;
+  for (int k = tid; k < H * half; k += 256) {
+    const int h = k / half, j = k - h * half;
+    const T* qr = q + (int64_t)t * q_tok + (int64_t)h * q_head + nope;
+    const float x1 = (float)qr[j], x2 = (float)qr[half + j];
+    const float co = c[j], si = c[half + j];
+    T* o = qf + (int64_t)t * qf_tok + (int64_t)h * qf_head + lat;
+    o[j] = (T)(x1 * co - x2 * si);
+    o[half + j] = (T)(x2 * co + x1 * si);
+  }
+  for (int k = tid; k < H * tail; k += 256) {
+    const int h = k / tail, j = k - h * tail;
+    qf[(int64_t)t * qf_tok + (int64_t)h * qf_head + lat + rope + j] = (T)0.f;
+  }
+}
+
+OME_API int ome_latent_prep(const void* a, int64_t lda, int qlr, int lat, int rope, const void* w, float eps,
+                            const int* pos, const float* cs, const int* slots, void* k_cache, void* v_cache, int D,
+                            int P, const void* q, int64_t q_tok, int64_t q_head, int nope, int H, void* qf,
+                            int64_t qf_tok, int64_t qf_head, int T, int f32, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (rope % 2 || lat <= 0 || H <= 0 || lat + rope > D || P <= 0) return -2;
+  if (f32)
+    latent_prep_kernel<float><<<T, 256, 0, stream>>>((const float*)a, lda, qlr, lat, rope, (const float*)w, eps, pos,
+                                                     cs, slots, (float*)k_cache, (float*)v_cache, D, P,
+                                                     (const float*)q, q_tok, q_head, nope, H, (float*)qf, qf_tok,
+                                                     qf_head);
+  else
+    latent_prep_kernel<bf16><<<T, 256, 0, stream>>>((const bf16*)a, lda, qlr, lat, rope, (const bf16*)w, eps, pos, cs,
+                                                    slots, (bf16*)k_cache, (bf16*)v_cache, D, P, (const bf16*)q,
+                                                    q_tok, q_head, nope, H, (bf16*)qf, qf_tok, qf_head);
+  return (int)hipGetLastError();
+}

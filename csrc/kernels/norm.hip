@@ -367,3 +367,150 @@ OME_API int ome_residual_rmsnorm(float* res, int64_t res_stride, const void* x1,
   OME_CHECK_LAUNCH();
   return 0;
 }
+
+// ------------------------------------------------------------------------------------------
+// Post-norm step of an fp32 residual stream: res += norm(y) * w (+ b), the norm taken over the
+// SUBLAYER OUTPUT y (not over the stream).  kind 0: layer norm ((y - mean) / sqrt(var + eps), var =
+// mean squared deviation), kind 1: RMS norm (y / sqrt(mean(y^2) + eps)).  Statistics, scaling and
+// the sum are fp32; `out` (optional) gets the updated stream rounded to T: the next GEMM's input.
+// One workgroup per row; the row of y stays in registers (H <= 256 * PN_MAX) or is re-read.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void post_norm_add_kernel(float* __restrict__ res, int64_t res_stride,
+                                                            const T* __restrict__ y, int64_t y_stride,
+                                                            const T* __restrict__ w, const T* __restrict__ b,
+                                                            T* __restrict__ out, int64_t out_stride, int H, float eps,
+                                                            int kind) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const T* yr = y + row * y_stride;
+  float* r = res + row * res_stride;
+  float s = 0.f;
+  if (kind == 0) {
+    for (int i = threadIdx.x; i < H; i += 256) s += (float)yr[i];
+    s = block_sum<256>(s, red);
+  }
+  const float mean = kind == 0 ? s / (float)H : 0.f;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float d = (float)yr[i] - mean;
+    ss += d * d;
+  }
+  ss = block_sum<256>(ss, red);
+  const float rs = 1.f / sqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += 256) {
+    float v = ((float)yr[i] - mean) * rs * (float)w[i];
+    if (b != nullptr) v += (float)b[i];
+    v += r[i];
+    r[i] = v;
+    if (out != nullptr) out[row * out_stride + i] = (T)v;
+  }
+}
+
+OME_API int ome_post_norm_add(float* res, int64_t res_stride, const void* y, int64_t y_stride, const void* w,
+                              const void* b, void* out, int64_t out_stride, int rows, int H, float eps, int kind,
+                              int f32, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0 || kind < 0 || kind > 1) return -2;
+  if (f32)
+    post_norm_add_kernel<float><<<rows, 256, 0, stream>>>(res, res_stride, (const float*)y, y_stride, (const float*)w,
+                                                          (const float*)b, (float*)out, out_stride, H, eps, kind);
+  else
+    post_norm_add_kernel<bf16><<<rows, 256, 0, stream>>>(res, res_stride, (const bf16*)y, y_stride, (const bf16*)w,
+                                                         (const bf16*)b, (bf16*)out, out_stride, H, eps, kind);
+  OME_CHECK_LAUNCH();
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// PolyNorm activation: out = a N(z) + b N(z^2) + c N(z^3) + e with element-wise powers and
+// N(u) = u / sqrt(mean(u^2) + eps) over the row; coef = (a, b, c, e) fp32.  The three mean
+// squares (of z, z^2, z^3) come from one pass in fp32, the second pass writes the sum.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void polynorm_kernel(const T* __restrict__ z, int64_t z_stride,
+                                                       const float* __restrict__ coef, T* __restrict__ out,
+                                                       int64_t out_stride, int F, float eps) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const T* zr = z + row * z_stride;
+  float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  for (int i = threadIdx.x; i < F; i += 256) {
+    const float v = (float)zr[i], v2 = v * v;
+    s1 += v2;
+    s2 += v2 * v2;
+    s3 += v2 * v2 * v2;
+  }
+  s1 = block_sum<256>(s1, red);
+  s2 = block_sum<256>(s2, red);
+  s3 = block_sum<256>(s3, red);
+  const float n = (float)F;
+  const float r1 = coef[0] / sqrtf(s1 / n + eps), r2 = coef[1] / sqrtf(s2 / n + eps),
+              r3 = coef[2] / sqrtf(s3 / n + eps), e = coef[3];
+  for (int i = threadIdx.x; i < F; i += 256) {
+    const float v = (float)zr[i];
+    out[row * out_stride + i] = (T)(v * (r1 + v * (r2 + v * r3)) + e);
+  }
+}
+
+OME_API int ome_polynorm(const void* z, int64_t z_stride, const float* coef, void* out, int64_t out_stride, int rows,
+                         int F, float eps, int f32, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (F <= 0) return -2;
+  if (f32)
+    polynorm_kernel<float><<<rows, 256, 0, stream>>>((const float*)z, z_stride, coef, (float*)out, out_stride, F, eps);
+  else
+    polynorm_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)z, z_stride, coef, (bf16*)out, out_stride, F, eps);
+  OME_CHECK_LAUNCH();
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Row norm for any width and element type: out = norm(x) * w (+ b), kind 0 layer norm / 1 RMS
+// norm, statistics in fp32.  TI: the input's type (an fp32 residual stream, or a projection's
+// output), TO: the type of w, b and out.  One workgroup per row.
+// ------------------------------------------------------------------------------------------
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void row_norm_kernel(const TI* __restrict__ x, int64_t x_stride,
+                                                       const TO* __restrict__ w, const TO* __restrict__ b,
+                                                       TO* __restrict__ out, int64_t out_stride, int H, float eps,
+                                                       int kind) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const TI* xr = x + row * x_stride;
+  float s = 0.f;
+  if (kind == 0) {
+    for (int i = threadIdx.x; i < H; i += 256) s += (float)xr[i];
+    s = block_sum<256>(s, red);
+  }
+  const float mean = kind == 0 ? s / (float)H : 0.f;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float d = (float)xr[i] - mean;
+    ss += d * d;
+  }
+  ss = block_sum<256>(ss, red);
+  const float rs = 1.f / sqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += 256) {
+    float v = ((float)xr[i] - mean) * rs * (float)w[i];
+    if (b != nullptr) v += (float)b[i];
+    out[row * out_stride + i] = (TO)v;
+  }
+}
+
+OME_API int ome_row_norm(const void* x, int64_t x_stride, int x_f32, const void* w, const void* b, void* out,
+                         int64_t out_stride, int rows, int H, float eps, int kind, int f32, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0 || kind < 0 || kind > 1 || (f32 && !x_f32)) return -2;
+  if (f32)
+    row_norm_kernel<float, float><<<rows, 256, 0, stream>>>((const float*)x, x_stride, (const float*)w,
+                                                            (const float*)b, (float*)out, out_stride, H, eps, kind);
+  else if (x_f32)
+    row_norm_kernel<float, bf16><<<rows, 256, 0, stream>>>((const float*)x, x_stride, (const bf16*)w, (const bf16*)b,
+                                                           (bf16*)out, out_stride, H, eps, kind);
+  else
+    row_norm_kernel<bf16, bf16><<<rows, 256, 0, stream>>>((const bf16*)x, x_stride, (const bf16*)w, (const bf16*)b,
+                                                          (bf16*)out, out_stride, H, eps, kind);
+  OME_CHECK_LAUNCH();
+  return 0;
+}

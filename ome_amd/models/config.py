@@ -141,23 +141,57 @@ def attn_tile_dim(d: int) -> int:
 
 
 def _layer_list_keys(c: dict[str, Any]) -> dict[str, Any]:
-    """Layer-list configs (``architecture: Zavilorn``): ``layers`` is a list of blocks, each with
-    its mixer ``type``, the mixer's own sizes and its feed-forward.  The standard keys describe the
-    envelope the runtime sizes its workspaces by (widest attention layer, fewest kv heads); the
-    model reads the per-layer entries from ``extra``."""
-    attn = [L["mixer"]["left"] for L in c["layers"] if L.get("type") == "parallel"]
-    ff = [L["mlp"]["ff"] for L in c["layers"] if L.get("mlp")]
-    D = max([attn_tile_dim(max(a["dim"], a["vdim"])) for a in attn] or [64])
+    """Layer-list configs (``architecture: Zavilorn`` / ``Metitar``): ``layers`` is a list of blocks,
+    each with its mixer ``type``, the mixer's own sizes and its feed-forward.  The standard keys
+    describe the envelope the runtime sizes its workspaces by (widest attention layer, fewest kv
+    heads); the model reads the per-layer entries from ``extra``."""
+    attn, dims = [], []
+    for L in c["layers"]:
+        m = L.get("mixer") or {}
+        if L.get("type") == "parallel":
+            attn.append(m["left"])
+            dims.append(attn_tile_dim(max(m["left"]["dim"], m["left"]["vdim"])))
+        elif L.get("type") == "latent_attention":   # absorbed form: one shared head of latent + rotary width
+            attn.append(m)
+            dims.append(attn_tile_dim(m["kv_rank"] + m["rot_dim"]))
+    ff = [(L["mlp"].get("ff") or (L["mlp"].get("expert") or {}).get("ff") or 0) for L in c["layers"] if L.get("mlp")]
+    D = max(dims or [64])
     out = dict(c)
     out.update(architectures=[c["architecture"]], model_type=c["architecture"].lower(),
                hidden_size=c["width"], vocab_size=c["vocab"], num_hidden_layers=len(c["layers"]),
                rms_norm_eps=(c.get("norm") or {}).get("eps", 1e-6), tie_word_embeddings=True,
                num_attention_heads=max([a["heads"] for a in attn] or [1]),
-               num_key_value_heads=min([a["kv_heads"] for a in attn] or [1]), head_dim=D,
+               num_key_value_heads=min([a.get("kv_heads", 1) for a in attn] or [1]), head_dim=D,
                intermediate_size=max(ff or [c["width"]]), rope_theta=(attn[0]["rot"]["base"] if attn else 10000.0),
                partial_rotary_factor=(attn[0]["rot"]["dims"] / D if attn else 1.0),
                max_position_embeddings=int(c.get("max_positions", 131072)), torch_dtype="bfloat16")
     return out
+
+
+def yarn_rope_table(base: float, rot_dim: int, max_pos: int, scaling: dict | None, device=None) -> torch.Tensor:
+    """[max_pos, rot_dim] fp32 (cos | sin) for rotary frequencies f_i = base^(-2i/rot_dim) under
+    YaRN scaling ``{factor, original, fast, slow}`` (None: unscaled): with dim(t) = rot_dim *
+    ln(original / (2 pi t)) / (2 ln base), lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)),
+    rot_dim - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), frequency i becomes
+    f_i / factor * ramp_i + f_i * (1 - ramp_i), and cos / sin are scaled by 0.1 ln(factor) + 1.
+    Built in fp64, stored fp32."""
+    i = torch.arange(0, rot_dim // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / rot_dim)
+    m = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def dim_of(t: float) -> float:
+            return rot_dim * math.log(orig / (2 * math.pi * t)) / (2 * math.log(float(base)))
+
+        lo = max(math.floor(dim_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(dim_of(float(scaling["slow"]))), rot_dim - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        m = 0.1 * math.log(factor) + 1.0
+    fr = torch.outer(torch.arange(max_pos, dtype=torch.float64), f)
+    cs = (torch.cat([fr.cos(), fr.sin()], -1) * m).float()
+    return cs.to(device) if device is not None else cs
 
 
 def plain_rope_table(base: float, rot_dim: int, max_pos: int, device=None) -> torch.Tensor:

@@ -7,7 +7,17 @@ constructor argument), for decoders that assemble their layers from a per-layer 
 * :class:`GatedDeltaMixer` -- the gated delta rule (short causal convolutions, unit-norm q / k,
   per-head decay and write strength, fp32 state per request slot);
 * :class:`Mamba2Mixer` -- Mamba-2 / SSD selective scan with grouped B / C and a gated group norm;
-* :class:`ClampedGLU` -- gated feed-forward ``min(g, L) * sigmoid(1.702 min(g, L)) * (clamp(u, -L, L) + 1)``.
+* :class:`ClampedGLU` -- gated feed-forward ``min(g, L) * sigmoid(1.702 min(g, L)) * (clamp(u, -L, L) + 1)``;
+* :class:`LatentAttention` -- multi-head latent attention (low-rank queries, one cached latent +
+  one shared rotary key per token, YaRN-scaled rotary table, a learned per-head softmax sink), run
+  absorbed as multi-query attention over the paged cache; a layer may read another layer's cache;
+* :class:`Hgrn2Mixer` -- HGRN2 gated linear recurrence (lower-bounded forget gate that also sets
+  the write strength, fp32 state per request slot, per-head RMS norm);
+* :class:`PolyNormMLP` -- two-matrix feed-forward with the PolyNorm activation;
+* :class:`InputScaledMoE` -- sigmoid-routed mixture of SwiGLU experts whose router score scales the
+  expert's input, plus an optional always-on shared expert;
+* :class:`TokenSideInput` -- a gated per-layer slice of a second token embedding, projected back to
+  the stream.
 
 Each block owns its weights (fused input projection, checkpoint tensors concatenated at load), its
 recurrent state (``alloc_state``) and one ``forward(h, ctx)`` over a varlen batch of rows: prompt
@@ -24,7 +34,7 @@ import torch
 
 from ome_amd import ops
 from ome_amd.models.common import AttnMeta, PagedKVCache, mixed_attention
-from ome_amd.models.config import attn_tile_dim, plain_rope_table
+from ome_amd.models.config import attn_tile_dim, plain_rope_table, yarn_rope_table
 from ome_amd.models.quant import linear
 
 
@@ -39,9 +49,10 @@ class MixerCtx:
 
 
 def paged_attention(q: torch.Tensor, k_cache, v_cache, meta: AttnMeta, scale: float, window: int = -1,
-                    keep_first: int = 0) -> torch.Tensor:
-    """Decode / prefill / mixed dispatch over the paged cache (q [T, Hq, D] -> [T, Hq, D])."""
-    kw = dict(window=window, keep_first=keep_first)
+                    keep_first: int = 0, sinks: torch.Tensor | None = None) -> torch.Tensor:
+    """Decode / prefill / mixed dispatch over the paged cache (q [T, Hq, D] -> [T, Hq, D]).
+    ``sinks``: fp32 [Hq] logits that join each head's softmax denominator (no key, no value)."""
+    kw = dict(window=window, keep_first=keep_first, sinks=sinks)
     if meta.is_decode:
         return ops.paged_decode(q, k_cache, v_cache, meta.block_tables, meta.seq_lens, scale, meta.decode_ws,
                                 order=meta.order, **kw)
@@ -240,3 +251,208 @@ class ClampedGLU(_Block):
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return linear(ops.act_and_mul(linear(h, self.w_gu), 2, limit=self.limit), self.w_d)
+
+
+class LatentAttention(_Block):
+    """Multi-head latent attention.  c_q = RMSNorm(W_dq h) w_dqn, q = W_uq c_q, laid out per head
+    as [``dim`` unrotated | ``rot_dim`` rotated]; W_dkv h = [``kv_rank`` latent | ``rot_dim`` shared
+    rotary key]; c = RMSNorm(latent) w_dkvn; per head k = [W_uk c | rope(k_pe)], v = W_uv c; score =
+    q . k * ``scale``; causal softmax whose denominator also holds exp(``sink``_h); W_o.  Rotary
+    pairs are (i, i + rot_dim/2) with the YaRN-scaled table of ``config.yarn_rope_table``.
+
+    Runs absorbed: q_lat = W_uk^T q_nope, so all heads share one key [c | rope(k_pe)] and one value
+    c per token -- multi-query attention over a paged cache of head width D = tile(kv_rank +
+    rot_dim) (``ops.latent_prep`` -> ``paged_attention`` -> W_uv per head).  ``kv_layer`` != ``layer``:
+    this layer has no W_dkv and attends over ``kv_layer``'s cache rows with its own W_uk / W_uv.
+    Checkpoint tensors ``dq dq.norm uq [dkv dkv.norm] uk uv sink o``."""
+
+    HEAD_GROUP = 16   # query heads per kv head one attention launch takes
+
+    def __init__(self, layer: int, kv_layer: int, width: int, heads: int, dim: int, rot_dim: int, vdim: int,
+                 kv_rank: int, q_rank: int, rot_base: float, rot_scaling: dict | None, scale: float, eps: float,
+                 max_positions: int, device, dtype):
+        super().__init__(device, dtype)
+        if rot_dim % 2 or rot_dim <= 0:
+            raise ValueError(f"latent attention: rotary width {rot_dim} must be even and positive")
+        self.layer, self.kv_layer, self.width, self.H = layer, kv_layer, width, heads
+        self.dim, self.rot, self.vdim, self.R, self.qr = dim, rot_dim, vdim, kv_rank, q_rank
+        self.scale, self.eps = float(scale), float(eps)
+        self.own_cache = kv_layer == layer
+        self.D = attn_tile_dim(kv_rank + rot_dim)
+        self.cos_sin = yarn_rope_table(rot_base, rot_dim, max_positions, rot_scaling, self.device)
+        self.w_in = self.qn = self.w_uq = self.kvn = self.w_uk = self.w_uv = self.sink = self.w_o = None
+
+    def load(self, t: dict) -> None:
+        H, R = self.H, self.R
+        self.w_in = self._put(torch.cat([t["dq"], t["dkv"]], 0) if self.own_cache else t["dq"])
+        self.qn, self.w_uq = self._put(t["dq.norm"]), self._put(t["uq"])
+        if self.own_cache:
+            self.kvn = self._put(t["dkv.norm"])
+        self.w_uk = self._put(t["uk"].view(H, self.dim, R))                       # q_lat = q_nope @ W_uk[h]
+        self.w_uv = self._put(t["uv"].view(H, self.vdim, R).transpose(1, 2))      # o = o_lat @ W_uv[h]^T
+        self.sink, self.w_o = self._put(t["sink"], torch.float32), self._put(t["o"])
+
+    def init_random(self, gen, std: float) -> None:
+        H, R = self.H, self.R
+        self.w_in = self._rand(gen, self.qr + (R + self.rot if self.own_cache else 0), self.width, std=std)
+        self.qn = torch.ones(self.qr, dtype=self.dtype, device=self.device)
+        self.w_uq = self._rand(gen, H * (self.dim + self.rot), self.qr, std=std)
+        if self.own_cache:
+            self.kvn = torch.ones(R, dtype=self.dtype, device=self.device)
+        self.w_uk, self.w_uv = self._rand(gen, H, self.dim, R, std=std), self._rand(gen, H, R, self.vdim, std=std)
+        self.sink = torch.zeros(H, dtype=torch.float32, device=self.device)
+        self.w_o = self._rand(gen, self.width, H * self.vdim, std=std)
+
+    def forward(self, h: torch.Tensor, ctx: MixerCtx) -> torch.Tensor:
+        T, H, R, D = h.shape[0], self.H, self.R, self.D
+        a = linear(h, self.w_in)                                          # [T, q_rank (| latent | k_pe)]
+        q = linear(ops.row_norm(a[:, :self.qr], self.qn, None, self.eps, 1), self.w_uq).view(T, H, self.dim + self.rot)
+        q_full = torch.empty(T, H, D, dtype=h.dtype, device=h.device)     # [W_uk^T q_nope | rope(q_pe) | 0]
+        k_cache, v_cache = ctx.kv.layer(self.kv_layer)
+        own = self.own_cache
+        ops.latent_prep(a, self.qr, R, self.rot, self.kvn, self.eps, ctx.meta.positions, self.cos_sin, ctx.meta.slots,
+                        k_cache if own else None, v_cache if own else None, q, self.dim, q_full)
+        torch.bmm(q[..., :self.dim].transpose(0, 1), self.w_uk, out=q_full[:, :, :R].transpose(0, 1))
+        G = self.HEAD_GROUP
+        if H <= G:
+            o_lat = paged_attention(q_full, k_cache, v_cache, ctx.meta, self.scale, sinks=self.sink)
+        else:   # the kernels share one kv head among at most G query heads: run the heads in groups
+            o_lat = torch.cat([paged_attention(q_full[:, g:g + G], k_cache, v_cache, ctx.meta, self.scale,
+                                               sinks=self.sink[g:g + G]) for g in range(0, H, G)], 1)
+        o = torch.empty(T, H * self.vdim, dtype=h.dtype, device=h.device)
+        torch.bmm(o_lat[:, :, :R].transpose(0, 1), self.w_uv, out=o.view(T, H, self.vdim).transpose(0, 1))
+        return linear(o, self.w_o)
+
+
+class Hgrn2Mixer(_Block):
+    """HGRN2.  q = silu(W_q h) (``heads`` x ``dim``), v = W_v h (``heads`` x ``vdim``), forget gate
+    f = l + (1 - l) sigmoid(W_f h + b_f) with the learned lower bound l; per head S <- diag(f) S +
+    (1 - f) v^T, o = S^T q (no key, no other scale); RMSNorm of each head's o with a shared weight
+    [vdim]; W_o.  Checkpoint tensors ``q f f.b lower v norm o``; state S [slots, heads, dim, vdim]
+    fp32.  Activations, gate, recurrence and norm are one kernel (``ops.hgrn2_scan``)."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, eps: float, device, dtype):
+        super().__init__(device, dtype)
+        self.width, self.H, self.dim, self.vdim, self.eps = width, heads, dim, vdim, float(eps)
+        self.w_in = self.f_bias = self.lower = self.gnorm = self.w_o = None
+        self.rec_state = None
+
+    def load(self, t: dict) -> None:
+        self.w_in = self._put(torch.cat([t["q"], t["f"], t["v"]], 0))
+        self.f_bias, self.lower = self._put(t["f.b"]), self._put(t["lower"])
+        self.gnorm, self.w_o = self._put(t["norm"]), self._put(t["o"])
+
+    def init_random(self, gen, std: float) -> None:
+        hd = self.H * self.dim
+        self.w_in = self._rand(gen, 2 * hd + self.H * self.vdim, self.width, std=std)
+        self.f_bias = torch.zeros(hd, dtype=self.dtype, device=self.device)
+        self.lower = torch.linspace(0.0, 0.9, hd, device=self.device).to(self.dtype)
+        self.gnorm = torch.ones(self.vdim, dtype=self.dtype, device=self.device)
+        self.w_o = self._rand(gen, self.width, self.H * self.vdim, std=std)
+
+    def alloc_state(self, slots: int) -> None:
+        self.rec_state = torch.zeros(slots, self.H, self.dim, self.vdim, dtype=torch.float32, device=self.device)
+
+    def forward(self, h: torch.Tensor, ctx: MixerCtx) -> torch.Tensor:
+        cu, slot, reset = ctx.seqs
+        hd = self.H * self.dim
+        p = linear(h, self.w_in)                                          # [T, q | f | v]
+        o = ops.hgrn2_scan(p[:, :hd], p[:, hd:2 * hd], p[:, 2 * hd:], self.f_bias, self.lower, self.gnorm,
+                           self.rec_state, cu, slot, reset, self.H, self.dim, self.vdim, self.eps)
+        return linear(o, self.w_o)
+
+
+class PolyNormMLP(_Block):
+    """W_down act(W_up h) with act(z) = a N(z) + b N(z^2) + c N(z^3) + e (element-wise powers, N =
+    division by the row's root mean square).  Checkpoint tensors ``up down act`` (act = a, b, c, e)."""
+
+    def __init__(self, width: int, ff: int, eps: float, device, dtype):
+        super().__init__(device, dtype)
+        self.width, self.ff, self.eps = width, ff, float(eps)
+        self.w_up = self.w_d = self.coef = None
+
+    def load(self, t: dict) -> None:
+        self.w_up, self.w_d, self.coef = self._put(t["up"]), self._put(t["down"]), self._put(t["act"], torch.float32)
+
+    def init_random(self, gen, std: float) -> None:
+        self.w_up, self.w_d = self._rand(gen, self.ff, self.width, std=std), self._rand(gen, self.width, self.ff,
+                                                                                        std=std)
+        self.coef = torch.tensor([1.0, 0.5, 0.25, 0.0], dtype=torch.float32, device=self.device)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return linear(ops.polynorm(linear(h, self.w_up), self.coef, self.eps), self.w_d)
+
+
+class InputScaledMoE(_Block):
+    """Mixture of SwiGLU experts (no biases): router scores s = sigmoid(W_r h) from fp32 logits, the
+    ``top`` largest chosen, weights = those scores (not renormalised) applied to the expert's INPUT:
+    y = sum_e expert_e(s_e h) (+ shared(h), an always-on expert of its own width).  Checkpoint
+    tensors ``router e<j>.gate|up|down [shared.gate|up|down]``.
+
+    Two paths: rows pre-scaled and expanded (``ops.scale_rows``), sorted by expert, through the
+    grouped MFMA GEMMs (bf16, widths that are multiples of 32); otherwise every expert over all
+    rows as batched library GEMMs with the unchosen rows' inputs zeroed (an expert without biases
+    maps 0 to 0, so they add nothing) -- any shape, any dtype, no host synchronisation either way."""
+
+    def __init__(self, width: int, experts: int, top: int, ff: int, shared_ff: int, device, dtype):
+        super().__init__(device, dtype)
+        self.width, self.E, self.k, self.ff, self.sff = width, experts, top, ff, int(shared_ff or 0)
+        self.w_router = self.w13 = self.w2 = self.w_sgu = self.w_sd = None
+        self._ones = None
+
+    def load(self, t: dict) -> None:
+        self.w_router = self._put(t["router"])
+        self.w13 = self._put(torch.stack([torch.cat([t[f"e{e}.gate"], t[f"e{e}.up"]], 0) for e in range(self.E)]))
+        self.w2 = self._put(torch.stack([t[f"e{e}.down"] for e in range(self.E)]))
+        if self.sff:
+            self.w_sgu, self.w_sd = self._put(torch.cat([t["shared.gate"], t["shared.up"]], 0)), self._put(t["shared.down"])
+
+    def init_random(self, gen, std: float) -> None:
+        self.w_router = self._rand(gen, self.E, self.width, std=std)
+        self.w13, self.w2 = self._rand(gen, self.E, 2 * self.ff, self.width, std=std), self._rand(
+            gen, self.E, self.width, self.ff, std=std)
+        if self.sff:
+            self.w_sgu, self.w_sd = self._rand(gen, 2 * self.sff, self.width, std=std), self._rand(
+                gen, self.width, self.sff, std=std)
+
+    def grouped_ok(self, h: torch.Tensor) -> bool:
+        return h.is_cuda and h.dtype == torch.bfloat16 and self.width % 32 == 0 and self.ff % 32 == 0
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        T, W = h.shape
+        logits = ops.lm_head_f32(h, self.w_router)                        # fp32 [T, E]
+        tw, tid = ops.moe_route(logits, self.k, False, "sigmoid")
+        sh = linear(ops.act_and_mul(linear(h, self.w_sgu), 0), self.w_sd) if self.sff else None
+        if self.grouped_ok(h):
+            y, inv = ops.moe_experts_sorted(ops.scale_rows(h, tw), tid.view(-1), self.w13, self.w2, 0, self.E)
+            if self._ones is None or self._ones.shape[0] < T:
+                self._ones = torch.ones(max(T, 256), self.k, dtype=torch.float32, device=h.device)
+            return ops._combine(y, self._ones[:T], inv, T, self.k, W, 1.0, sh.contiguous() if sh is not None else None)
+        wd = torch.zeros(T, self.E, dtype=torch.float32, device=h.device).scatter_(1, tid.long(), tw)
+        xe = (wd.t()[:, :, None] * h.float()[None]).to(h.dtype)           # [E, T, W]: s_e h, or 0
+        gu = torch.bmm(xe, self.w13.transpose(1, 2))
+        hh = ops.act_and_mul(gu.view(self.E * T, 2 * self.ff), 0).view(self.E, T, self.ff)
+        y = torch.bmm(hh, self.w2.transpose(1, 2)).float().sum(0)
+        return (y if sh is None else y + sh.float()).to(h.dtype)
+
+
+class TokenSideInput(_Block):
+    """Per-layer token input: e = the layer's ``dim``-wide slice of a second embedding row of the
+    token; g = gelu_tanh(W_gate x) * e; y = W_proj g.  The caller adds RMSNorm(y) * ``norm`` to the
+    stream.  Checkpoint tensors ``gate proj norm`` (the table is shared by all layers)."""
+
+    def __init__(self, width: int, dim: int, col0: int, device, dtype):
+        super().__init__(device, dtype)
+        self.width, self.dim, self.col0 = width, dim, col0
+        self.w_gate = self.w_proj = self.norm = None
+
+    def load(self, t: dict) -> None:
+        self.w_gate, self.w_proj, self.norm = self._put(t["gate"]), self._put(t["proj"]), self._put(t["norm"])
+
+    def init_random(self, gen, std: float) -> None:
+        self.w_gate, self.w_proj = self._rand(gen, self.dim, self.width, std=std), self._rand(gen, self.width, self.dim,
+                                                                                              std=std)
+        self.norm = torch.ones(self.width, dtype=self.dtype, device=self.device)
+
+    def forward(self, h: torch.Tensor, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+        return linear(ops.gelu_gather_mul(linear(h, self.w_gate), ids, table, self.col0), self.w_proj)

@@ -804,10 +804,10 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, ws: DecodeW
     B, Hq, D = q.shape
     Hkv, P = k_cache.shape[1], k_cache.shape[2]
     if q.dtype == torch.float32:   # fp32 models: the exact fp32 kernel (row b = sequence b at its last position)
-        _f32_only(softcap, sinks, alibi, row_lo, blocksparse)
+        _f32_only(softcap, alibi, row_lo, blocksparse)
         return _paged_attention_f32(q, k_cache, v_cache, block_tables,
                                     torch.arange(B, dtype=torch.int32, device=q.device), _i32(seq_lens) - 1, scale,
-                                    window, keep_first, out)
+                                    window, keep_first, out, sinks)
     if ws is None:
         ws = DecodeWorkspace(B, Hq, D, block_tables.shape[1] * P, device=q.device)
     out = torch.empty_like(q) if out is None else out
@@ -821,14 +821,16 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, ws: DecodeW
     return out
 
 
-def _f32_only(softcap, sinks, alibi, rows, blocksparse) -> None:
-    if softcap or sinks is not None or alibi is not None or rows is not None or blocksparse is not None:
-        raise NotImplementedError("fp32 attention: plain / windowed causal masks only")
+def _f32_only(softcap, alibi, rows, blocksparse) -> None:
+    if softcap or alibi is not None or rows is not None or blocksparse is not None:
+        raise NotImplementedError("fp32 attention: plain / windowed causal masks (with sinks) only")
 
 
-def _paged_attention_f32(q, k_cache, v_cache, block_tables, row_seq, row_pos, scale, window, keep_first, out):
+def _paged_attention_f32(q, k_cache, v_cache, block_tables, row_seq, row_pos, scale, window, keep_first, out,
+                         sinks=None):
     """fp32 paged attention (``attention_f32.hip``): q [T, Hq, D] fp32, fp32 caches; row t belongs
-    to block-table row ``row_seq[t]`` and sits at absolute position ``row_pos[t]`` (< 0: padding)."""
+    to block-table row ``row_seq[t]`` and sits at absolute position ``row_pos[t]`` (< 0: padding).
+    ``sinks``: fp32 [Hq] logits that join the softmax denominator."""
     T, Hq, D = q.shape
     Hkv, P = k_cache.shape[1], k_cache.shape[2]
     assert k_cache.dtype == v_cache.dtype == torch.float32 and q.stride(2) == 1 and q.stride(1) == D
@@ -837,7 +839,7 @@ def _paged_attention_f32(q, k_cache, v_cache, block_tables, row_seq, row_pos, sc
     call("ome_paged_attention_f32", q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
          _i32(block_tables).data_ptr(), block_tables.stride(0), _i32(row_seq.contiguous()).data_ptr(),
          _i32(row_pos.contiguous()).data_ptr(), out.data_ptr(), out.stride(0), T, Hq, Hkv, D, P, float(scale),
-         int(window), int(keep_first), stream_ptr())
+         int(window), int(keep_first), _sinks(sinks), stream_ptr())
     return out
 
 
@@ -1570,12 +1572,12 @@ def paged_prefill(q, k_cache, v_cache, block_tables, cu_q, kv_lens, items, scale
     Tq, Hq, D = q.shape
     Hkv, P = k_cache.shape[1], k_cache.shape[2]
     if q.dtype == torch.float32:   # fp32 models: the exact fp32 kernel, one (sequence, position) per row
-        _f32_only(softcap, sinks, alibi, row_hi, blocksparse)
+        _f32_only(softcap, alibi, row_hi, blocksparse)
         r = torch.arange(Tq, dtype=torch.int64, device=q.device)
         seq = torch.bucketize(r, _i32(cu_q)[1:].long(), right=True).clamp_(max=cu_q.shape[0] - 2)
         pos = _i32(kv_lens)[seq] - cu_q[seq + 1] + r
         return _paged_attention_f32(q, k_cache, v_cache, block_tables, seq.to(torch.int32), pos.to(torch.int32),
-                                    scale, window, keep_first, out)
+                                    scale, window, keep_first, out, sinks)
     out = torch.empty_like(q) if out is None else out
     rows = 32
     if isinstance(items, PrefillPlan):
@@ -1691,4 +1693,142 @@ def pool(hidden: torch.Tensor, cu_lens: torch.Tensor, mode: int = 0, normalize: 
     out = torch.empty(S, H, dtype=torch.float32, device=hidden.device)
     call("ome_pool", hidden.data_ptr(), _i32(cu_lens).data_ptr(), out.data_ptr(), S, H, mode, int(normalize),
          stream_ptr())
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# Post-norm fp32 residual streams, residual convolution, latent-attention glue, HGRN2, PolyNorm
+# ---------------------------------------------------------------------------------------------
+def post_norm_add(res: torch.Tensor, y: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None, eps: float,
+                  kind: int = 0, out_dtype=None):
+    """Post-norm step of an fp32 residual stream, in place: ``res += norm(y) * w (+ b)`` with the
+    norm over the sublayer OUTPUT ``y`` (kind 0: layer norm, 1: RMS norm; statistics and sum in
+    fp32).  Returns the updated stream rounded to ``out_dtype`` (the next GEMM's input), or None."""
+    if not _gpu(res):
+        return ref.post_norm_add(res, y, w, b, eps, kind, out_dtype)
+    T, H = res.shape
+    assert res.dtype == torch.float32 and res.stride(1) == 1 and y.shape == res.shape and y.stride(1) == 1
+    f32 = _f32(y, w, b)
+    out = torch.empty(T, H, dtype=out_dtype, device=res.device) if out_dtype is not None else None
+    assert out is None or out.dtype == y.dtype
+    call("ome_post_norm_add", res.data_ptr(), res.stride(0), y.data_ptr(), y.stride(0), w.data_ptr(), ptr(b),
+         ptr(out), H if out is not None else 0, T, H, float(eps), int(kind), f32, stream_ptr())
+    return out
+
+
+def conv_mix(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor, cu, slot, reset, out_dtype) -> torch.Tensor:
+    """``x + causal_conv(x)`` per channel over a varlen batch of an fp32 stream: x [T, C] fp32, taps
+    w [C, K] (tap K-1 on the current row, no bias, no activation), ``state`` [slots, C, K-1] fp32 =
+    the last K-1 input rows of each sequence, continued / updated (``reset[s]``: start from zeros)."""
+    T, C = x.shape
+    out = torch.empty(T, C, dtype=out_dtype, device=x.device)
+    if not _gpu(x):
+        return ref.conv_mix(x, w, state, cu, slot, reset, out)
+    assert x.dtype == torch.float32 and state.dtype == torch.float32 and x.stride(1) == 1
+    assert w.is_contiguous() and state.is_contiguous() and state.shape[1:] == (C, w.shape[1] - 1)
+    call("ome_conv_mix", x.data_ptr(), x.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0), state.data_ptr(),
+         _i32(cu).data_ptr(), _i32(slot).data_ptr(), _i32(reset).data_ptr(), slot.shape[0], T, C, w.shape[1],
+         _f32(w, out), stream_ptr())
+    return out
+
+
+def latent_prep(a: torch.Tensor, qlr: int, lat: int, rope: int, w: torch.Tensor | None, eps: float,
+                positions: torch.Tensor, cos_sin: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor | None,
+                v_cache: torch.Tensor | None, q: torch.Tensor, nope: int, q_full: torch.Tensor) -> None:
+    """Latent attention before the paged attention kernels, in its absorbed (multi-query) form:
+    from the fused down projection ``a`` [T, qlr + lat + rope] write the token's key
+    ``[RMSNorm(c) * w | RoPE(k_pe)]`` into ``k_cache`` [pages, 1, P, D] and its value
+    ``RMSNorm(c) * w`` into ``v_cache`` [pages, 1, D, P] (D >= lat + rope; the tails stay zero),
+    and the rotated q_pe of every head into ``q_full[:, :, lat:lat + rope]`` (zeros up to D);
+    q [T, H, nope + rope].  Rotary pairs are (j, j + rope/2); ``cos_sin`` fp32 [positions, rope] =
+    cos | sin.  ``k_cache`` None: only the queries (a layer that reads another layer's cache)."""
+    if not _gpu(q):
+        return ref.latent_prep(a, qlr, lat, rope, w, eps, positions, cos_sin, slots, k_cache, v_cache, q, nope, q_full)
+    T, H = q.shape[0], q.shape[1]
+    D = q_full.shape[2]
+    P = 1
+    if k_cache is not None:
+        P = k_cache.shape[2]
+        assert k_cache.shape[1] == 1 and k_cache.shape[3] == D and v_cache.shape[1:] == (1, D, P)
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and a.stride(1) == 1
+    f32 = _f32(q, q_full, k_cache, v_cache, w, a if k_cache is not None else None)
+    assert q.stride(2) == 1 and q_full.stride(2) == 1
+    assert cos_sin.dtype == torch.float32 and cos_sin.shape[1] == rope and cos_sin.is_contiguous()
+    call("ome_latent_prep", a.data_ptr(), a.stride(0), qlr, lat, rope, ptr(w), float(eps), _i32(positions).data_ptr(),
+         cos_sin.data_ptr(), _i32(slots).data_ptr(), ptr(k_cache), ptr(v_cache), D, P, q.data_ptr(), q.stride(0),
+         q.stride(1), nope, H, q_full.data_ptr(), q_full.stride(0), q_full.stride(1), T, f32, stream_ptr())
+
+
+def hgrn2_scan(q: torch.Tensor, f: torch.Tensor, v: torch.Tensor, f_bias: torch.Tensor, lower: torch.Tensor,
+               w: torch.Tensor, state: torch.Tensor, cu, slot, reset, H: int, dim: int, vdim: int,
+               eps: float) -> torch.Tensor:
+    """HGRN2 recurrence with its activations and output norm: q' = silu(q), gate g = lower +
+    (1 - lower) * sigmoid(f + f_bias); per head S <- diag(g) S + (1 - g) v^T, o = S^T q'; returns
+    RMSNorm_vdim(o) * w as [T, H * vdim].  q / f [T, H * dim] and v [T, H * vdim] are views of one
+    projection output (same row stride); ``state`` [slots, H, dim, vdim] fp32 is continued /
+    updated per sequence (``cu`` / ``slot`` / ``reset`` as in :func:`ssm_conv1d`)."""
+    T = q.shape[0]
+    out = torch.empty(T, H * vdim, dtype=q.dtype, device=q.device)
+    if not _gpu(q):
+        return ref.hgrn2_scan(q, f, v, f_bias, lower, w, state, cu, slot, reset, H, dim, vdim, eps, out)
+    assert q.stride(0) == f.stride(0) == v.stride(0) and q.stride(1) == f.stride(1) == v.stride(1) == 1
+    assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, dim, vdim)
+    assert f_bias.is_contiguous() and lower.is_contiguous() and w.is_contiguous()
+    call("ome_hgrn2_scan", q.data_ptr(), f.data_ptr(), v.data_ptr(), q.stride(0), f_bias.data_ptr(),
+         lower.data_ptr(), w.data_ptr(), state.data_ptr(), out.data_ptr(), out.stride(0), _i32(cu).data_ptr(),
+         _i32(slot).data_ptr(), _i32(reset).data_ptr(), slot.shape[0], H, dim, vdim, float(eps),
+         _f32(q, f, v, f_bias, lower, w), stream_ptr())
+    return out
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """PolyNorm activation over rows: ``a N(z) + b N(z^2) + c N(z^3) + e`` (element-wise powers,
+    N(u) = u / sqrt(mean(u^2) + eps)); ``coef`` = fp32 (a, b, c, e)."""
+    out = torch.empty(z.shape, dtype=z.dtype, device=z.device)
+    if not _gpu(z):
+        return ref.polynorm(z, coef, eps, out)
+    assert z.stride(1) == 1 and coef.dtype == torch.float32 and coef.numel() == 4 and coef.is_contiguous()
+    call("ome_polynorm", z.data_ptr(), z.stride(0), coef.data_ptr(), out.data_ptr(), out.stride(0), z.shape[0],
+         z.shape[1], float(eps), _f32(z), stream_ptr())
+    return out
+
+
+def gelu_gather_mul(g: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: int) -> torch.Tensor:
+    """``gelu_tanh(g) * table[ids, col0 : col0 + n]`` for g [T, n]: a projection gated against a
+    slice of a per-token embedding row."""
+    out = torch.empty(g.shape, dtype=g.dtype, device=g.device)
+    if not _gpu(g):
+        return ref.gelu_gather_mul(g, ids, table, col0, out)
+    n = g.shape[1]
+    assert g.stride(1) == 1 and table.stride(1) == 1 and 0 <= col0 and col0 + n <= table.shape[1]
+    call("ome_gelu_gather_mul", g.data_ptr(), g.stride(0), _i32(ids).data_ptr(), table.data_ptr(), table.stride(0),
+         table.shape[0], int(col0), out.data_ptr(), g.shape[0], n, _f32(g, table), stream_ptr())
+    return out
+
+
+def scale_rows(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x [T, H], w fp32 [T, k] -> [T * k, H] rows ``w[t, j] * x[t]`` (fp32 product, one rounding):
+    the expanded inputs of a mixture of experts whose router weight scales the expert's input."""
+    T, H = x.shape
+    k = w.shape[1]
+    if not _gpu(x):
+        return (x.float()[:, None, :] * w.float()[:, :, None]).to(x.dtype).reshape(T * k, H)
+    assert x.stride(1) == 1 and w.dtype == torch.float32 and w.is_contiguous()
+    out = torch.empty(T * k, H, dtype=x.dtype, device=x.device)
+    call("ome_scale_rows", x.data_ptr(), x.stride(0), w.data_ptr(), k, out.data_ptr(), T, H, _f32(x), stream_ptr())
+    return out
+
+
+def row_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None, eps: float, kind: int = 1) -> torch.Tensor:
+    """``norm(x) * w (+ b)`` over rows of any width: kind 0 layer norm, 1 RMS norm; x fp32 (a
+    residual stream) or w's dtype, possibly a row-strided view; statistics in fp32, result in w's
+    dtype."""
+    if not _gpu(x):
+        return ref.row_norm(x, w, b, eps, kind)
+    assert x.dim() == 2 and x.stride(1) == 1 and w.is_contiguous()
+    f32 = _f32(w, b)
+    assert x.dtype == torch.float32 or x.dtype == w.dtype
+    out = torch.empty(x.shape, dtype=w.dtype, device=x.device)
+    call("ome_row_norm", x.data_ptr(), x.stride(0), int(x.dtype == torch.float32), w.data_ptr(), ptr(b),
+         out.data_ptr(), out.stride(0), x.shape[0], x.shape[1], float(eps), int(kind), f32, stream_ptr())
     return out

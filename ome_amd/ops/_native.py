@@ -44,7 +44,16 @@ _SIGNATURES = {
                                      i32, i32, i32, i32, i32, i32, i32, vp],
         "ome_head_gate": [vp, vp, i64, vp, i32, i32, i32, i32, i32, i32, vp],
         "ome_paged_attention_f32": [vp, i64, vp, vp, vp, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, f32, i32,
-                                    i32, vp],
+                                    i32, vp, vp],
+        "ome_post_norm_add": [vp, i64, vp, i64, vp, vp, vp, i64, i32, i32, f32, i32, i32, vp],
+        "ome_row_norm": [vp, i64, i32, vp, vp, vp, i64, i32, i32, f32, i32, i32, vp],
+        "ome_polynorm": [vp, i64, vp, vp, i64, i32, i32, f32, i32, vp],
+        "ome_gelu_gather_mul": [vp, i64, vp, vp, i64, i32, i32, vp, i32, i32, i32, vp],
+        "ome_scale_rows": [vp, i64, vp, i32, vp, i32, i32, i32, vp],
+        "ome_conv_mix": [vp, i64, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
+        "ome_latent_prep": [vp, i64, i32, i32, i32, vp, f32, vp, vp, vp, vp, vp, i32, i32, vp, i64, i64, i32, i32, vp,
+                            i64, i64, i32, i32, vp],
+        "ome_hgrn2_scan": [vp, vp, vp, i64, vp, vp, vp, vp, vp, i64, vp, vp, vp, i32, i32, i32, i32, f32, i32, vp],
         "ome_act": [vp, i64, i32, vp],
         "ome_ssm_conv1d": [vp, i64, vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, vp],
         "ome_dyn_conv1d": [vp, i64, vp, i64, i32, vp, i64, vp, vp, vp, vp, i32, i32, i32, vp],

@@ -652,3 +652,106 @@ def mla_attn(q, cache, block_tables, tok_row, kv_lens, scale, dv=512):
         s = (q[t].float() @ kv.t()) * scale
         out[t] = (torch.softmax(s, -1) @ kv[:, :dv]).to(q.dtype)
     return out
+
+
+# ---------------------------------------------------------------------------------------------
+# Post-norm residual streams, residual convolutions, latent attention glue, HGRN2, PolyNorm
+# ---------------------------------------------------------------------------------------------
+def post_norm_add(res, y, w, b, eps, kind, out_dtype):
+    yf = y.float()
+    if kind == 0:
+        yf = yf - yf.mean(-1, keepdim=True)
+    n = yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    if b is not None:
+        n = n + b.float()
+    res.add_(n)
+    return res.to(out_dtype) if out_dtype is not None else None
+
+
+def conv_mix(x, w, state, cu, slot, reset, out):
+    K = w.shape[1]
+    wf = w.float()
+    for s in range(len(slot)):
+        r0, r1 = int(cu[s]), int(cu[s + 1])
+        if r1 <= r0:
+            continue
+        st = state[int(slot[s])]                                      # [C, K-1]
+        prev = torch.zeros_like(st) if int(reset[s]) else st
+        seq = torch.cat([prev.t(), x[r0:r1]], 0)                      # [K-1+L, C] fp32
+        acc = x[r0:r1].clone()
+        for j in range(K):
+            acc += wf[:, j] * seq[j:j + r1 - r0]
+        out[r0:r1] = acc.to(out.dtype)
+        if K > 1:
+            st.copy_(seq[-(K - 1):].t())
+    return out
+
+
+def latent_prep(a, qlr, lat, rope, w, eps, positions, cos_sin, slots, k_cache, v_cache, q, nope, q_full):
+    cs = cos_sin.index_select(0, positions.long())
+    half = rope // 2
+
+    def rot(x, cos, sin):
+        x1, x2 = x[..., :half].float(), x[..., half:].float()
+        return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], -1).to(x.dtype)
+
+    if k_cache is not None:
+        P, D = k_cache.shape[2], k_cache.shape[3]
+        ckv = a[:, qlr:qlr + lat + rope]
+        cf = ckv[:, :lat].float()
+        c = (cf * torch.rsqrt(cf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(a.dtype)
+        sl = slots.long().clamp_min(0)
+        k_cache.view(-1, D)[sl, :lat + rope] = torch.cat([c, rot(ckv[:, lat:], cs[:, :half], cs[:, half:])], -1)
+        v_cache[sl // P, 0, :lat, sl % P] = c
+    q_full[:, :, lat:lat + rope] = rot(q[..., nope:], cs[:, None, :half], cs[:, None, half:])
+    q_full[:, :, lat + rope:] = 0
+
+
+def hgrn2_scan(q, f, v, f_bias, lower, w, state, cu, slot, reset, H, dim, vdim, eps, out):
+    lo = lower.float().view(H, dim)
+    for s in range(len(slot)):
+        r0, r1 = int(cu[s]), int(cu[s + 1])
+        if r1 <= r0:
+            continue
+        S = state[int(slot[s])]                                       # [H, dim, vdim] fp32
+        if int(reset[s]):
+            S.zero_()
+        L = r1 - r0
+        qs = torch.nn.functional.silu(q[r0:r1].float()).view(L, H, dim)
+        fs = lo + (1 - lo) * torch.sigmoid(f[r0:r1].float().view(L, H, dim) + f_bias.float().view(H, dim))
+        vs = v[r0:r1].float().view(L, H, vdim)
+        o = torch.empty(L, H, vdim)
+        for t in range(L):
+            S.copy_(fs[t][..., None] * (S - vs[t][:, None, :]) + vs[t][:, None, :])
+            o[t] = torch.einsum("hdv,hd->hv", S, qs[t])
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        out[r0:r1] = o.reshape(L, H * vdim).to(out.dtype)
+    return out
+
+
+def polynorm(z, coef, eps, out):
+    zf = z.float()
+    a, b, c, e = (float(x) for x in coef)
+
+    def n(u):
+        return u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)
+
+    out.copy_((a * n(zf) + b * n(zf * zf) + c * n(zf * zf * zf) + e).to(out.dtype))
+    return out
+
+
+def gelu_gather_mul(g, ids, table, col0, out):
+    n = g.shape[1]
+    e = table[ids.long().clamp(0, table.shape[0] - 1), col0:col0 + n].float()
+    out.copy_((torch.nn.functional.gelu(g.float(), approximate="tanh") * e).to(out.dtype))
+    return out
+
+
+def row_norm(x, w, b, eps, kind):
+    xf = x.float()
+    if kind == 0:
+        xf = xf - xf.mean(-1, keepdim=True)
+    n = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    if b is not None:
+        n = n + b.float()
+    return n.to(w.dtype)
