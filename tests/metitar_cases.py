@@ -31,7 +31,7 @@ def config_a():
 def config_b():
     """Other sizes and the values the first config keeps apart made equal, 1 or absent: HGRN2
     first, dim = vdim = rot_dim, one head, two taps, no rotary scaling, every expert chosen (top =
-    experts), no shared expert, unit scales, two attention layers with caches of their own and
+    experts), no shared expert, unit logit scale, two attention layers with caches of their own and
     different widths, one of them read by a third."""
     return mo.make_config([
         mo.hgrn2_layer(heads=1, dim=8, vdim=8, mlp=mo.dense(17)),
@@ -42,7 +42,7 @@ def config_b():
                            mlp=mo.dense(33)),
         mo.attention_layer(heads=2, dim=8, rot_dim=8, vdim=4, kv_rank=8, q_rank=3, base=7.0, scaling=None, scale=0.5,
                            kv_from=1, mlp=None),
-    ], width=40, vocab=37, embed_scale=1.0, eps=1e-6, taps=2, side=2, logit_scale=1.0)
+    ], width=40, vocab=37, embed_scale=2.0, eps=1e-6, taps=2, side=2, logit_scale=1.0)
 
 
 def config_c():
@@ -63,24 +63,24 @@ def config_bf16():
 
 
 def prompts(cfg, weights, lengths, seed=1, min_margin=0.0, cache=None):
-    """Random prompts; with ``min_margin`` > 0 the seed is advanced until every router decision of
-    every prompt has at least that margin in the oracle (a 16-bit run may otherwise pick another
+    """Random prompts; with ``min_margin`` > 0 each prompt's seed is advanced until every router
+    decision on it has at least that margin in the oracle (a 16-bit run may otherwise pick another
     expert on a near tie, which is no fault).  Oracle logits land in ``cache``."""
-    for s in range(seed, seed + 200):
-        g = random.Random(s)
-        ps = [[g.randrange(cfg["vocab"]) for _ in range(n)] for n in lengths]
-        ok = True
-        for p in ps:
+    out = []
+    for k, n in enumerate(lengths):
+        for s in range(200):
+            g = random.Random(1000 * (seed + s) + k)
+            p = [g.randrange(cfg["vocab"]) for _ in range(n)]
             m: list = []
             want = mo.forward(cfg, weights, p, margins=m)
-            if cache is not None:
-                cache[tuple(p)] = want
-            if m and min(m) < min_margin:
-                ok = False
+            if not m or min(m) >= min_margin:
+                if cache is not None:
+                    cache[tuple(p)] = want
+                out.append(p)
                 break
-        if ok:
-            return ps
-    raise AssertionError("no prompt set with the wanted router margin")
+        else:
+            raise AssertionError("no prompt with the wanted router margin")
+    return out
 
 
 def assert_matches_oracle(eng, cfg, weights, toks: dict, schedule, tol, oracle_cache=None):
