@@ -59,7 +59,7 @@ def config_bf16():
         mo.hgrn2_layer(heads=2, dim=16, vdim=8, mlp=mo.dense(40)),
         mo.attention_layer(heads=2, dim=8, rot_dim=8, vdim=16, kv_rank=24, q_rank=12, kv_from=0, mlp=mo.moe(2, 1, 32, 32)),
         mo.hgrn2_layer(heads=3, dim=8, vdim=24, mlp=None),
-    ], width=64, vocab=61, taps=4, side=8)
+    ], width=64, vocab=61, taps=4, side=8, embed_scale=8.0)
 
 
 def prompts(cfg, weights, lengths, seed=1, min_margin=0.0, cache=None):
@@ -83,9 +83,12 @@ def prompts(cfg, weights, lengths, seed=1, min_margin=0.0, cache=None):
     return out
 
 
-def assert_matches_oracle(eng, cfg, weights, toks: dict, schedule, tol, oracle_cache=None):
+def assert_matches_oracle(eng, cfg, weights, toks: dict, schedule, tol, oracle_cache=None, typical=None):
+    """Every position within ``tol`` of the oracle.  ``typical`` (16-bit runs): also the median over
+    all positions -- the design's output norms amplify 16-bit rounding at single positions of a small
+    random model, while a fault of the cache, the state or a mask moves most positions by far more."""
     got = replay(eng, toks, schedule)
-    worst = 0.0
+    worst, every = 0.0, []
     for rid, t in toks.items():
         key = tuple(t)
         if oracle_cache is not None and key in oracle_cache:
@@ -94,9 +97,14 @@ def assert_matches_oracle(eng, cfg, weights, toks: dict, schedule, tol, oracle_c
             want = mo.forward(cfg, weights, t)
             if oracle_cache is not None:
                 oracle_cache[key] = want
-        err = mo.logit_error(got[rid], want)
+        errs = mo.logit_errors(got[rid], want)
+        every.append(errs)
+        err = errs.max().item()
         worst = max(worst, err)
         assert err < tol, f"request {rid} ({len(t)} tokens): logits differ from the oracle by {err:.3g} (limit {tol})"
+    if typical is not None:
+        med = torch.cat(every).median().item()
+        assert med < typical, f"median difference from the oracle {med:.3g} (limit {typical})"
     return worst
 
 
@@ -143,7 +151,7 @@ def attention_block(m, width, dev, dt, eps=1e-5, max_pos=512, pages=96):
     return blk, PagedKVCache(1, pages, 1, blk.D, 16, dt, dev)
 
 
-def planted_key_case(dev, dt, tol, n, i, j, cuts, seen=True):
+def planted_key_case(dev, dt, tol, n, i, j, cuts, seen=True, row_only=False):
     """A key made to dominate query i's softmax whenever it is visible.  The latent's first half
     reads the input's first half and feeds the keys, its second half reads the input's second half
     and feeds the values; q's unrotated part is tied to k's (same down projection, norm weight and
@@ -151,7 +159,9 @@ def planted_key_case(dev, dt, tol, n, i, j, cuts, seen=True):
     half has the query's own key direction but a value of its own; its second half is small, which
     makes its normalised latent (and so its score) larger than the query's own.  Losing (or wrongly
     seeing) that one key among hundreds moves the output by much more than the tolerance.
-    ``seen`` False: j > i lies in the future of query i and must leave its output alone."""
+    ``seen`` False: j > i lies in the future of query i and must leave its output alone.
+    ``row_only``: compare row i alone (16-bit runs: the other rows' softmaxes are as sharp but
+    between random keys, where rounding of the scores decides)."""
     W, R, r, d = 64, 32, 4, 32
     m = mo.attention_layer(heads=2, dim=d, rot_dim=r, vdim=8, kv_rank=R, q_rank=R, scale=0.5)["mixer"]
     w = mo.sub(mo.random_weights(mo.make_config([{"type": "latent_attention", "mixer": m, "mlp": None}], width=W), 21),
@@ -176,7 +186,8 @@ def planted_key_case(dev, dt, tol, n, i, j, cuts, seen=True):
     blk, kv = attention_block(m, W, dev, dt, pages=2 * (n // 16 + 2) + 8)
     blk.load(w)
     got = run_chunks(blk, h.to(device=dev, dtype=dt), cuts, kv).cpu()
-    rel = ((got.to(F64) - want).abs().max() / want.abs().max()).item()
+    rows = slice(i, i + 1) if row_only else slice(None)
+    rel = ((got.to(F64) - want)[rows].abs().max() / want[rows].abs().max()).item()
     assert rel < tol, rel
     if seen:    # the planted key carries the answer: hidden, the oracle's row i moves
         moved = mo.latent_attention(hq, w64, m, 1e-5, hide=(i, j))

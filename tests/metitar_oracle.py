@@ -231,14 +231,16 @@ def make_config(layers, width=24, vocab=53, embed_scale=3.0, eps=1e-5, taps=3, s
     return cfg
 
 
-def random_weights(cfg, seed=0):
-    """bf16 tensors under the checkpoint's names; scales chosen so that every branch matters."""
+def random_weights(cfg, seed=0, gain=1.0):
+    """bf16 tensors under the checkpoint's names; scales chosen so that every branch matters
+    (``gain`` < 1 flattens every projection: a smoother model for 16-bit runs, whose rounding a
+    stack of output norms otherwise amplifies)."""
     g = torch.Generator().manual_seed(seed)
     W, V, n = cfg["width"], cfg["vocab"], len(cfg["layers"])
     bf = torch.bfloat16
 
     def mat(o, i, s=1.0):
-        return (torch.randn(o, i, generator=g) * s / math.sqrt(i)).to(bf)
+        return (torch.randn(o, i, generator=g) * s * gain / math.sqrt(i)).to(bf)
 
     def vec(k, lo, hi):
         return (torch.rand(k, generator=g) * (hi - lo) + lo).to(bf)
@@ -273,7 +275,7 @@ def random_weights(cfg, seed=0):
                 t[q + "up"], t[q + "down"] = mat(f["ff"], W, 2.0), mat(W, f["ff"], 2.0)
                 t[q + "act"] = torch.tensor([0.9, -0.5, 0.4, 0.1]).to(bf)
             else:
-                t[q + "router"] = mat(f["router"]["experts"], W, 0.3)   # (scores stay off saturation)
+                t[q + "router"] = mat(f["router"]["experts"], W, 0.3 / gain)   # (scores off saturation; not flattened)
                 names = [f"e{e}." for e in range(f["router"]["experts"])] + (["shared."] if f.get("shared") else [])
                 for nm in names:
                     ff = f["shared"]["ff"] if nm == "shared." else f["expert"]["ff"]
@@ -294,11 +296,15 @@ def save_model(folder, cfg, weights):
     return str(folder)
 
 
-def logit_error(got, want):
-    """Root mean square over the vocabulary of the centred difference, relative to the rms of the
-    oracle's centred logits."""
+def logit_errors(got, want):
+    """Per position: root mean square over the vocabulary of the centred difference, relative to the
+    rms of the oracle's centred logits."""
     got, want = got.to(F64), want.to(F64)
     d = got - want
     d = d - d.mean(-1, keepdim=True)
     ref = want - want.mean(-1, keepdim=True)
-    return (d.pow(2).mean(-1).sqrt() / ref.pow(2).mean().sqrt()).max().item()
+    return d.pow(2).mean(-1).sqrt() / ref.pow(2).mean().sqrt()
+
+
+def logit_error(got, want):
+    return logit_errors(got, want).max().item()
