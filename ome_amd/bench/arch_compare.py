@@ -1,4 +1,12 @@
-"""Zavilorn beside the closest existing hybrid (NemotronH: Mamba-2 + attention + dense MLP) at equal
+"""Layer-list designs beside their closest existing model at equal size (``bench.py --arch-compare
+[--arch-design zavilorn|metitar]``).
+
+Metitar (latent attention + HGRN2, PolyNorm / input-scaled MoE feed-forwards) stands beside a
+DeepSeek-V2-style stack (multi-head latent attention, dense then routed feed-forwards with shared
+experts) of the same width, depth, head count, latent width and expert sizes; its kernel table sets
+every kernel added for the design next to the like kernel of the existing models.
+
+Zavilorn beside the closest existing hybrid (NemotronH: Mamba-2 + attention + dense MLP) at equal
 width, depth and mixer sizes, random weights: engine-level prefill / decode throughput, and a
 per-kernel table that sets every kernel added for the design next to the like kernel of the
 existing models with its share of the HBM roofline (``bench.py --arch-compare``).
@@ -44,6 +52,46 @@ def nemotron_config(s: dict) -> dict:
                 head_dim=128, intermediate_size=s["ff"], mlp_hidden_act="relu2", mamba_num_heads=s["mheads"],
                 mamba_head_dim=64, ssm_state_size=128, n_groups=8, conv_kernel=4, vocab_size=s["vocab"],
                 layer_norm_epsilon=1e-6, max_position_embeddings=8192, time_step_min=0.001, tie_word_embeddings=True)
+
+
+M_SIZES = {
+    "2k": dict(width=2048, heads=16, q_rank=768, ff=5632, experts=32, top=4, eff=1024, sff=2048, vocab=32768),
+    "4k": dict(width=4096, heads=32, q_rank=1536, ff=14336, experts=32, top=4, eff=2048, sff=4096, vocab=32768),
+}
+
+
+def metitar_config(s: dict) -> dict:
+    """[latent attention + dense, hgrn2 + moe, hgrn2 + dense, latent attention on layer 0's cache + moe] x 2:
+    128 + 32-wide heads over a 224-wide latent (256-wide cache rows), HGRN2 heads of 128 x 128."""
+    att = {"heads": s["heads"], "dim": 128, "rot_dim": 32, "vdim": 128, "kv_rank": 224, "q_rank": s["q_rank"],
+           "rot": {"base": 10000.0, "dims": 32, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}},
+           "scale": 160 ** -0.5}
+    rec = {"heads": s["heads"], "dim": 128, "vdim": 128}
+    dense = {"kind": "dense", "ff": s["ff"]}
+    moe = {"kind": "moe", "router": {"experts": s["experts"], "top": s["top"]}, "expert": {"ff": s["eff"]},
+           "shared": {"ff": s["sff"]}}
+    layers = []
+    for blk in range(2):
+        a0 = 4 * blk
+        layers += [{"type": "latent_attention", "mixer": dict(att), "mlp": dense},
+                   {"type": "hgrn2", "mixer": rec, "mlp": moe}, {"type": "hgrn2", "mixer": rec, "mlp": dense},
+                   {"type": "latent_attention", "mixer": dict(att, kv_from=a0), "mlp": moe}]
+    return {"architecture": "Metitar", "embedding": {"scale": 4.0}, "layers": layers, "norm": {"eps": 1e-6},
+            "canon": {"taps": 4}, "token_side": {"dim": 64}, "logit_scale": 1.0, "vocab": s["vocab"],
+            "width": s["width"], "max_positions": 8192}
+
+
+def deepseek_like_config(s: dict) -> dict:
+    """Eight MLA layers (256 + 32-wide latent cache rows: the kernel's second shape), four dense then
+    four routed feed-forwards of the Metitar stack's sizes."""
+    return dict(architectures=["DeepseekV2ForCausalLM"], model_type="deepseek_v2", hidden_size=s["width"],
+                num_hidden_layers=8, num_attention_heads=s["heads"], num_key_value_heads=s["heads"],
+                intermediate_size=s["ff"], moe_intermediate_size=s["eff"], n_routed_experts=s["experts"],
+                n_shared_experts=s["sff"] // s["eff"], num_experts_per_tok=s["top"], first_k_dense_replace=4, n_group=1,
+                topk_group=1, topk_method="greedy", scoring_func="softmax", norm_topk_prob=False,
+                routed_scaling_factor=1.0, kv_lora_rank=256, q_lora_rank=s["q_rank"], qk_nope_head_dim=128,
+                qk_rope_head_dim=32, v_head_dim=128, vocab_size=s["vocab"], rms_norm_eps=1e-6, rope_theta=10000.0,
+                max_position_embeddings=8192, tie_word_embeddings=False)
 
 
 def _engine(name: str, cfg: dict, max_running: int, context: int):
@@ -193,8 +241,150 @@ def kernel_table(T: int = 4096, B: int = 64, ctx: int = 4096, width: int = 4096)
     return rows
 
 
-def run(sizes=("2k", "4k"), kernels: bool = True, only: str | None = None) -> dict:
+def kernel_table_metitar(T: int = 4096, B: int = 64, ctx: int = 4096, width: int = 4096) -> list[dict]:
+    """Metitar's kernels beside their like kernels (same columns as :func:`kernel_table`)."""
+    from ome_amd import ops
+    from ome_amd.models.config import yarn_rope_table
+    from ome_amd.models.mixers import InputScaledMoE
+
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def pair(name, new, like, bytes_new, bytes_like, note=""):
+        tn, tl = _time_us(new), _time_us(like)
+        fn, fl = bytes_new / tn / 1e3 / HBM_GBS, bytes_like / tl / 1e3 / HBM_GBS
+        rows.append({"kernel": name, "us": round(tn, 1), "roofline": round(fn, 3), "like_us": round(tl, 1),
+                     "like_roofline": round(fl, 3), "vs_like": round(fl / max(fn, 1e-9), 2), "note": note})
+
+    def seqs(lens):
+        cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32, device=dev)
+        n = len(lens)
+        return cu, torch.arange(n, dtype=torch.int32, device=dev), torch.zeros(n, dtype=torch.int32, device=dev)
+
+    torch.manual_seed(0)
+    H, d, vd = 32, 128, 128
+    for R, tag, lens in ((T, "prefill", [T // 8] * 8), (B, "decode", [1] * B)):
+        cu, slot, reset = seqs(lens)
+        S = len(lens)
+        # ---- post-norm residual add (fp32 stream, layer norm of the addend) vs add + RMSNorm on a bf16 stream
+        res = torch.randn(R, width, device=dev)
+        y = torch.randn(R, width, device=dev).to(bf)
+        w, b = torch.ones(width, device=dev, dtype=bf), torch.zeros(width, device=dev, dtype=bf)
+        rb, xb = res.to(bf), y.clone()
+        pair(f"post_norm_add layer norm ({tag})", lambda: ops.post_norm_add(res, y, w, b, 1e-6, 0, bf),
+             lambda: ops.fused_add_rmsnorm(xb, rb, w, 1e-6), R * width * 12, R * width * 8,
+             "fp32 stream: 12 B / element against 8; the addend is read twice more from cache (mean, variance)")
+        # ---- residual causal conv on the fp32 stream vs the conv + SiLU of the recurrent mixers
+        wc = (torch.randn(width, 4, device=dev) * 0.3).to(bf)
+        st32 = torch.zeros(S, width, 3, device=dev)
+        stb = torch.zeros(S, width, 3, device=dev, dtype=bf)
+        pair(f"conv_mix 4 taps ({tag})", lambda: ops.conv_mix(res, wc, st32, cu, slot, reset, bf),
+             lambda: ops.ssm_conv1d(y, wc, None, stb, cu, slot, reset), R * width * 6, R * width * 4,
+             "time-parallel tiles; like: one thread per channel walks the sequence")
+        # ---- HGRN2 scan (+ activations + head norm) vs the gated delta rule scan of equal head shape
+        p = torch.randn(R, 2 * H * d + H * vd, device=dev).to(bf)
+        fb, lo, gw = torch.zeros(H * d, device=dev, dtype=bf), torch.full((H * d,), 0.3, device=dev, dtype=bf), \
+            torch.ones(vd, device=dev, dtype=bf)
+        st = torch.zeros(S, H, d, vd, device=dev)
+        ab = torch.randn(R, 2 * H, device=dev).to(bf)
+        Al, db = torch.zeros(H, device=dev), torch.zeros(H, device=dev)
+        state_b = S * H * d * vd * 4 * 2
+        io_new, io_like = R * (2 * H * d + 2 * H * vd) * 2, R * (2 * H * d + 2 * H * vd + 2 * H) * 2
+        pair(f"hgrn2_scan 32 x 128 x 128 ({tag})",
+             lambda: ops.hgrn2_scan(p[:, :H * d], p[:, H * d:2 * H * d], p[:, 2 * H * d:], fb, lo, gw, st, cu, slot, reset,
+                                    H, d, vd, 1e-6),
+             lambda: ops.gdn_scan(p[:, :H * d], p[:, H * d:2 * H * d], p[:, 2 * H * d:], ab[:, :H], ab[:, H:], Al, db, st,
+                                  cu, slot, reset, H, H), state_b + io_new, state_b + io_like,
+             "like: Qwen3-Next's gated delta rule (state in and out dominate decode; prefill is latency of the walk)")
+        # ---- PolyNorm vs SiLU-and-mul
+        I = 14336
+        z = torch.randn(R, I, device=dev).to(bf)
+        gu = torch.randn(R, 2 * I, device=dev).to(bf)
+        coef = torch.tensor([0.9, -0.4, 0.3, 0.05], device=dev)
+        pair(f"polynorm ({tag})", lambda: ops.polynorm(z, coef, 1e-6), lambda: ops.act_and_mul(gu, 0), R * I * 4,
+             R * I * 6, "two passes over the row (three mean squares, then the sum)")
+        # ---- latent glue vs the MLA glue
+        qlr, lat, rope, D, P = 1536, 224, 32, 256, 16
+        a = torch.randn(R, qlr + lat + rope, device=dev).to(bf)
+        a2 = torch.randn(R, qlr + 256 + rope, device=dev).to(bf)
+        nw, nw2 = torch.ones(lat, device=dev, dtype=bf), torch.ones(256, device=dev, dtype=bf)
+        pos = torch.arange(R, dtype=torch.int32, device=dev) % 2048
+        slots = torch.arange(R, dtype=torch.int32, device=dev) + P
+        cs = yarn_rope_table(10000.0, rope, 2048, None, dev)
+        q = torch.randn(R, H, 128 + rope, device=dev).to(bf)
+        kc = torch.zeros(R // P + 2, 1, P, D, device=dev, dtype=bf)
+        vc = torch.zeros(R // P + 2, 1, D, P, device=dev, dtype=bf)
+        qf = torch.empty(R, H, D, device=dev, dtype=bf)
+        lc = torch.zeros((R // P + 2) * P, 288, device=dev, dtype=bf)
+        qf2 = torch.empty(R, H, 288, device=dev, dtype=bf)
+        nb = R * ((lat + rope) * 2 * 2 + H * rope * 2 * 2)
+        pair(f"latent_prep ({tag})",
+             lambda: ops.latent_prep(a, qlr, lat, rope, nw, 1e-6, pos, cs, slots, kc, vc, q, 128, qf),
+             lambda: ops.mla_prep(a2, qlr, 256, rope, nw2, 1e-6, pos, cs, slots, lc, q, 128, qf2), nb + R * lat * 2, nb,
+             "writes the latent twice (key row, value column)")
+        # ---- routed feed-forward, router score on the expert's input vs on its output
+        E, k, ff = 32, 4, 2048
+        moe = InputScaledMoE(width, E, k, ff, 0, dev, bf)
+        moe.init_random(torch.Generator(device=dev).manual_seed(1), 0.02)
+        x = torch.randn(R, width, device=dev).to(bf)
+        lg = torch.randn(R, E, device=dev)
+        tw, tid = ops.moe_route(lg, k, False, "sigmoid")
+        touched = min(E, R * k) * 3 * ff * width * 2
+        pair(f"input-scaled moe 32 experts top 4 ({tag})", lambda: moe.forward(x),
+             lambda: ops.fused_moe(x, tw, tid, moe.w13, moe.w2, 0, 1.0), touched, touched,
+             "new: router GEMM + route + row scaling + grouped GEMMs + unit-weight combine; like: grouped GEMMs + combine")
+    # ---- latent attention, decode: multi-query over 256-wide cache rows with sinks vs the MLA kernel
+    Hq, D, P = 16, 256, 16
+    per = ctx // P
+    kc = (torch.randn(B * per + 1, 1, P, D, device=dev) * 0.3).to(bf)
+    vc = (torch.randn(B * per + 1, 1, D, P, device=dev) * 0.3).to(bf)
+    lc = (torch.randn(B * per + 1, P, 288, device=dev) * 0.3).to(bf)
+    bt = (torch.arange(B * per, dtype=torch.int32, device=dev) + 1).view(B, per)
+    sl = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+    q = torch.randn(B, Hq, D, device=dev).to(bf)
+    q2 = torch.randn(B, Hq, 288, device=dev).to(bf)
+    sinks = torch.zeros(Hq, device=dev)
+    ws = ops.DecodeWorkspace(B, Hq, D, ctx, 0, dev, parts=16)
+    mws = ops.MLAWorkspace(dev)
+    rows_i = torch.arange(B, dtype=torch.int32, device=dev)
+    pair("latent attention decode 64 x 4096 ctx, 16 heads",
+         lambda: ops.paged_decode(q, kc, vc, bt, sl, 0.08, ws, sinks=sinks),
+         lambda: ops.mla_attn(q2, lc, bt, rows_i, sl, 0.08, mws, dv=256), B * ctx * 256 * 2, B * ctx * 288 * 2,
+         "bytes that must move = the latent once; this path reads it as key and again as value")
+    # ---- latent attention, prefill 2 x 2048 rows
+    q_lens = [2048, 2048]
+    Tq = sum(q_lens)
+    qp = torch.randn(Tq, Hq, D, device=dev).to(bf)
+    qp2 = torch.randn(Tq, Hq, 288, device=dev).to(bf)
+    cu = torch.tensor([0, 2048, 4096], dtype=torch.int32, device=dev)
+    kl = torch.tensor(q_lens, dtype=torch.int32, device=dev)
+    bt2 = (torch.arange(2 * 128, dtype=torch.int32, device=dev) + 1).view(2, 128)
+    items = torch.tensor(ops.prefill_work_items(q_lens, q_lens), dtype=torch.int32, device=dev)
+    tok_row = torch.arange(Tq, dtype=torch.int32, device=dev) // 2048
+    tok_len = (torch.arange(Tq, dtype=torch.int32, device=dev) % 2048 + 1).to(torch.int32)
+    fl_new = 2.0 * Hq * (256 + 256) * sum(i + 1 for i in range(2048)) * 2
+    fl_like = 2.0 * Hq * (288 + 256) * sum(i + 1 for i in range(2048)) * 2
+    tn = _time_us(lambda: ops.paged_prefill(qp, kc, vc, bt2, cu, kl, items, 0.08, sinks=sinks), 10)
+    tl = _time_us(lambda: ops.mla_attn(qp2, lc, bt2, tok_row, tok_len, 0.08, mws, dv=256), 10)
+    rn, rl = fl_new / tn / 1e6 / 2.5e3, fl_like / tl / 1e6 / 2.5e3
+    rows.append({"kernel": "latent attention prefill 2 x 2048 rows, 16 heads", "us": round(tn, 1), "roofline": round(rn, 3),
+                 "like_us": round(tl, 1), "like_roofline": round(rl, 3), "vs_like": round(rl / max(rn, 1e-9), 2),
+                 "note": "share of 2.5 PFLOP/s bf16; like: the MLA kernel on 288-wide rows"})
+    return rows
+
+
+def run(sizes=("2k", "4k"), kernels: bool = True, only: str | None = None, design: str = "zavilorn") -> dict:
     out = {"throughput": [], "kernels": []}
+    if design == "metitar":
+        for k in sizes:
+            s = M_SIZES[k]
+            if only in (None, "metitar"):
+                out["throughput"].append(throughput(f"metitar-{k}", metitar_config(s)))
+            if only in (None, "deepseek"):
+                out["throughput"].append(throughput(f"deepseek-like-{k}", deepseek_like_config(s)))
+        if kernels:
+            out["kernels"] = kernel_table_metitar()
+        return out
     for k in sizes:
         s = SIZES[k]
         if only in (None, "zavilorn"):
@@ -212,9 +402,12 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--sizes", default="2k,4k")
     ap.add_argument("--no-kernels", action="store_true")
-    ap.add_argument("--only", choices=["zavilorn", "nemotron"], default=None, help="one stack (for kernel traces)")
+    ap.add_argument("--only", choices=["zavilorn", "nemotron", "metitar", "deepseek"], default=None,
+                    help="one stack (for kernel traces)")
+    ap.add_argument("--design", choices=["zavilorn", "metitar"], default="zavilorn")
+    ap.add_argument("--no-throughput", action="store_true", help="the kernel table only")
     a = ap.parse_args(argv)
-    res = run(tuple(a.sizes.split(",")), not a.no_kernels, a.only)
+    res = run(() if a.no_throughput else tuple(a.sizes.split(",")), not a.no_kernels, a.only, a.design)
     for r in res["throughput"]:
         print(json.dumps(r))
     for r in res["kernels"]:
