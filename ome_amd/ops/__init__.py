@@ -1774,12 +1774,14 @@ def hgrn2_scan(q: torch.Tensor, f: torch.Tensor, v: torch.Tensor, f_bias: torch.
     assert q.stride(0) == f.stride(0) == v.stride(0) and q.stride(1) == f.stride(1) == v.stride(1) == 1
     assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, dim, vdim)
     assert f_bias.is_contiguous() and lower.is_contiguous() and w.is_contiguous()
-    if vdim > 256 or -(-dim // max(1, min(256 // vdim, dim))) > 128:
+    vc = 32 if vdim >= 64 else vdim
+    if -(-dim // max(1, min(256 // vc, dim))) > 128:
         raise ValueError(f"hgrn2_scan: head state {dim} x {vdim} exceeds the register-resident kernel "
-                         "(vdim <= 256, dim / (256 // vdim) <= 128)")
+                         "(at most 128 state rows per thread)")
+    scratch = torch.empty(T, H * vdim, dtype=torch.float32, device=q.device)   # o before the head norm
     call("ome_hgrn2_scan", q.data_ptr(), f.data_ptr(), v.data_ptr(), q.stride(0), f_bias.data_ptr(),
-         lower.data_ptr(), w.data_ptr(), state.data_ptr(), out.data_ptr(), out.stride(0), _i32(cu).data_ptr(),
-         _i32(slot).data_ptr(), _i32(reset).data_ptr(), slot.shape[0], H, dim, vdim, float(eps),
+         lower.data_ptr(), w.data_ptr(), state.data_ptr(), scratch.data_ptr(), out.data_ptr(), T,
+         _i32(cu).data_ptr(), _i32(slot).data_ptr(), _i32(reset).data_ptr(), slot.shape[0], H, dim, vdim, float(eps),
          _f32(q, f, v, f_bias, lower, w), stream_ptr())
     return out
 

@@ -53,7 +53,7 @@ _SIGNATURES = {
         "ome_conv_mix": [vp, i64, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
         "ome_latent_prep": [vp, i64, i32, i32, i32, vp, f32, vp, vp, vp, vp, vp, i32, i32, vp, i64, i64, i32, i32, vp,
                             i64, i64, i32, i32, vp],
-        "ome_hgrn2_scan": [vp, vp, vp, i64, vp, vp, vp, vp, vp, i64, vp, vp, vp, i32, i32, i32, i32, f32, i32, vp],
+        "ome_hgrn2_scan": [vp, vp, vp, i64, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, f32, i32, vp],
         "ome_act": [vp, i64, i32, vp],
         "ome_ssm_conv1d": [vp, i64, vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, vp],
         "ome_dyn_conv1d": [vp, i64, vp, i64, i32, vp, i64, vp, vp, vp, vp, i32, i32, i32, vp],
