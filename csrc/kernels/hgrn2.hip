@@ -121,7 +121,9 @@ OME_API int ome_hgrn2_scan(const void* q, const void* f, const void* v, int64_t 
                            int f32, hipStream_t stream) {
   if (S <= 0 || H <= 0 || rows <= 0) return 0;
   if (dim <= 0 || vdim <= 0) return -2;
-  const int VC = vdim >= 64 ? 32 : vdim;
+  int VC = vdim >= 64 ? 32 : vdim;
+  // few long sequences: narrower slices, so that at least ~2 workgroups per CU walk them
+  while (VC > 8 && VC % 2 == 0 && (int64_t)H * ((vdim + VC - 1) / VC) * S < 512) VC /= 2;
   const int VS = (vdim + VC - 1) / VC;
   int G = 256 / VC;
   if (G > dim) G = dim;
@@ -136,6 +138,7 @@ OME_API int ome_hgrn2_scan(const void* q, const void* f, const void* v, int64_t 
                                                        reset, H, dim, vdim, VC, VS, G)
 #define HGRN2_ROWS(TT)                     \
   if (nr <= 4) HGRN2_LAUNCH(TT, 4);        \
+  else if (nr <= 8) HGRN2_LAUNCH(TT, 8);   \
   else if (nr <= 16) HGRN2_LAUNCH(TT, 16); \
   else if (nr <= 32) HGRN2_LAUNCH(TT, 32); \
   else if (nr <= 64) HGRN2_LAUNCH(TT, 64); \

@@ -398,7 +398,6 @@ class InputScaledMoE(_Block):
         super().__init__(device, dtype)
         self.width, self.E, self.k, self.ff, self.sff = width, experts, top, ff, int(shared_ff or 0)
         self.w_router = self.w13 = self.w2 = self.w_sgu = self.w_sd = None
-        self._ones = None
 
     def load(self, t: dict) -> None:
         self.w_router = self._put(t["router"])
@@ -425,9 +424,9 @@ class InputScaledMoE(_Block):
         sh = linear(ops.act_and_mul(linear(h, self.w_sgu), 0), self.w_sd) if self.sff else None
         if self.grouped_ok(h):
             y, inv = ops.moe_experts_sorted(ops.scale_rows(h, tw), tid.view(-1), self.w13, self.w2, 0, self.E)
-            if self._ones is None or self._ones.shape[0] < T:
-                self._ones = torch.ones(max(T, 256), self.k, dtype=torch.float32, device=h.device)
-            return ops._combine(y, self._ones[:T], inv, T, self.k, W, 1.0, sh.contiguous() if sh is not None else None)
+            ones = torch.ones(T, self.k, dtype=torch.float32, device=h.device)   # (per call: a buffer kept across
+            # calls would be pinned into captured decode graphs and could not grow afterwards)
+            return ops._combine(y, ones, inv, T, self.k, W, 1.0, sh.contiguous() if sh is not None else None)
         wd = torch.zeros(T, self.E, dtype=torch.float32, device=h.device).scatter_(1, tid.long(), tw)
         xe = (wd.t()[:, :, None] * h.float()[None]).to(h.dtype)           # [E, T, W]: s_e h, or 0
         gu = torch.bmm(xe, self.w13.transpose(1, 2))

@@ -1774,7 +1774,7 @@ def hgrn2_scan(q: torch.Tensor, f: torch.Tensor, v: torch.Tensor, f_bias: torch.
     assert q.stride(0) == f.stride(0) == v.stride(0) and q.stride(1) == f.stride(1) == v.stride(1) == 1
     assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, dim, vdim)
     assert f_bias.is_contiguous() and lower.is_contiguous() and w.is_contiguous()
-    vc = 32 if vdim >= 64 else vdim
+    vc = 32 if vdim >= 64 else vdim          # (the widest column slice the launcher picks)
     if -(-dim // max(1, min(256 // vc, dim))) > 128:
         raise ValueError(f"hgrn2_scan: head state {dim} x {vdim} exceeds the register-resident kernel "
                          "(at most 128 state rows per thread)")

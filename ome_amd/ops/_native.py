@@ -155,7 +155,7 @@ def load(name: str = "ome_kernels") -> C.CDLL:
             if os.environ.get("OME_AUTOBUILD", "1") == "1":
                 from ome_amd import build as _b
 
-                _b.build(verbose=False)
+                _b.build(verbose=False, only=(name,))   # (only the library asked for)
             if not path.exists():
                 raise NativeError(f"{path} missing — run `python -m ome_amd.build` (hipcc, gfx950)")
         lib = C.CDLL(str(path), mode=C.RTLD_GLOBAL)
