@@ -20,14 +20,14 @@
 
 namespace {
 
-constexpr int TB = 16;
+constexpr int TB_MAX = 16;   // rows per pair of barriers (fewer when a wide head's gates would not fit in LDS)
 
 template <typename T, int MAXR>
 __global__ __launch_bounds__(256) void hgrn2_scan_kernel(
     const T* __restrict__ q, const T* __restrict__ f, const T* __restrict__ v, int64_t in_stride,
     const T* __restrict__ f_bias, const T* __restrict__ lower, float* __restrict__ state, float* __restrict__ o,
     const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ reset, int H, int dim,
-    int vdim, int VC, int VS, int G) {
+    int vdim, int VC, int VS, int G, int TB) {
   extern __shared__ float sm[];
   float2* fq = (float2*)sm;                      // [TB][dim]
   float* vv = sm + 2 * TB * dim;                 // [TB][VC]
@@ -129,13 +129,15 @@ OME_API int ome_hgrn2_scan(const void* q, const void* f, const void* v, int64_t 
   if (G > dim) G = dim;
   const int nr = (dim + G - 1) / G;
   if (nr > 128) return -3;
+  int TB = rows <= S ? 1 : TB_MAX;   // (decode: every sequence is one row)
+  while (TB > 1 && sizeof(float) * (size_t)TB * (2 * dim + VC + G * VC) > 48 * 1024) TB /= 2;
   const size_t lds = sizeof(float) * (size_t)TB * (2 * dim + VC + G * VC);
-  if (lds > 64 * 1024 || (int64_t)H * VS > 65535 * 16 || S > 65535) return -4;
+  if (lds > 64 * 1024 || S > 65535) return -4;
   dim3 grid(H * VS, S);
 #define HGRN2_LAUNCH(TT, R)                                                                                       \
   hgrn2_scan_kernel<TT, R><<<grid, 256, lds, stream>>>((const TT*)q, (const TT*)f, (const TT*)v, in_stride,       \
                                                        (const TT*)f_bias, (const TT*)lower, state, o, cu, slot,  \
-                                                       reset, H, dim, vdim, VC, VS, G)
+                                                       reset, H, dim, vdim, VC, VS, G, TB)
 #define HGRN2_ROWS(TT)                     \
   if (nr <= 4) HGRN2_LAUNCH(TT, 4);        \
   else if (nr <= 8) HGRN2_LAUNCH(TT, 8);   \

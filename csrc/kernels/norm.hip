@@ -407,11 +407,103 @@ __global__ __launch_bounds__(256) void post_norm_add_kernel(float* __restrict__ 
   }
 }
 
+// bf16 rows of 8-element vectors held in registers (NCH vectors per thread): y is read once, with
+// 16-byte loads; the fp32 stream is read and written as float4 pairs.
+template <int NCH>
+__global__ __launch_bounds__(256) void post_norm_add_vec_kernel(float* __restrict__ res, int64_t res_stride,
+                                                                const bf16* __restrict__ y, int64_t y_stride,
+                                                                const bf16* __restrict__ w, const bf16* __restrict__ b,
+                                                                bf16* __restrict__ out, int64_t out_stride, int H,
+                                                                float eps, int kind) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const int nv = H >> 3;
+  const bf16* yr = y + row * y_stride;
+  float v[NCH][8];
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NCH; ++k) {
+    const int c = threadIdx.x + k * 256;
+    if (c < nv) {
+      const bf16x8 t = *(const bf16x8*)(yr + c * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[k][j] = (float)t[j];
+        s += v[k][j];
+      }
+    }
+  }
+  float mean = 0.f;
+  if (kind == 0) mean = block_sum<256>(s, red) / (float)H;
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NCH; ++k) {
+    if (threadIdx.x + k * 256 < nv) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[k][j] -= mean;
+        ss += v[k][j] * v[k][j];
+      }
+    }
+  }
+  ss = block_sum<256>(ss, red);
+  const float rs = 1.f / sqrtf(ss / (float)H + eps);
+  float* r = res + row * res_stride;
+#pragma unroll
+  for (int k = 0; k < NCH; ++k) {
+    const int c = threadIdx.x + k * 256;
+    if (c < nv) {
+      const bf16x8 wv = *(const bf16x8*)(w + c * 8);
+      f32x4 r0 = *(const f32x4*)(r + c * 8), r1 = *(const f32x4*)(r + c * 8 + 4);
+      float o[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = v[k][j] * rs * (float)wv[j];
+      if (b != nullptr) {
+        const bf16x8 bv = *(const bf16x8*)(b + c * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] += (float)bv[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        r0[j] += o[j];
+        r1[j] += o[j + 4];
+      }
+      *(f32x4*)(r + c * 8) = r0;
+      *(f32x4*)(r + c * 8 + 4) = r1;
+      if (out != nullptr) {
+        bf16x8 ov;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          ov[j] = (bf16)r0[j];
+          ov[j + 4] = (bf16)r1[j];
+        }
+        *(bf16x8*)(out + row * out_stride + c * 8) = ov;
+      }
+    }
+  }
+}
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
 OME_API int ome_post_norm_add(float* res, int64_t res_stride, const void* y, int64_t y_stride, const void* w,
                               const void* b, void* out, int64_t out_stride, int rows, int H, float eps, int kind,
                               int f32, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (H <= 0 || kind < 0 || kind > 1) return -2;
+  if (!f32 && H % 8 == 0 && H <= 8 * 256 * 8 && res_stride % 4 == 0 && y_stride % 8 == 0 && out_stride % 8 == 0 &&
+      aligned16(res) && aligned16(y) && aligned16(w) && aligned16(b) && aligned16(out)) {
+    const int nch = (H / 8 + 255) / 256;
+#define PNA_VEC(N)                                                                                                 \
+  post_norm_add_vec_kernel<N><<<rows, 256, 0, stream>>>(res, res_stride, (const bf16*)y, y_stride, (const bf16*)w, \
+                                                        (const bf16*)b, (bf16*)out, out_stride, H, eps, kind)
+    if (nch <= 1) PNA_VEC(1);
+    else if (nch <= 2) PNA_VEC(2);
+    else if (nch <= 4) PNA_VEC(4);
+    else PNA_VEC(8);
+#undef PNA_VEC
+    OME_CHECK_LAUNCH();
+    return 0;
+  }
   if (f32)
     post_norm_add_kernel<float><<<rows, 256, 0, stream>>>(res, res_stride, (const float*)y, y_stride, (const float*)w,
                                                           (const float*)b, (float*)out, out_stride, H, eps, kind);
@@ -453,10 +545,69 @@ __global__ __launch_bounds__(256) void polynorm_kernel(const T* __restrict__ z, 
   }
 }
 
+template <int NCH>
+__global__ __launch_bounds__(256) void polynorm_vec_kernel(const bf16* __restrict__ z, int64_t z_stride,
+                                                           const float* __restrict__ coef, bf16* __restrict__ out,
+                                                           int64_t out_stride, int F, float eps) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const int nv = F >> 3;
+  const bf16* zr = z + row * z_stride;
+  bf16x8 v[NCH];
+  float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+#pragma unroll
+  for (int k = 0; k < NCH; ++k) {
+    const int c = threadIdx.x + k * 256;
+    if (c < nv) {
+      v[k] = *(const bf16x8*)(zr + c * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float x = (float)v[k][j], x2 = x * x;
+        s1 += x2;
+        s2 += x2 * x2;
+        s3 += x2 * x2 * x2;
+      }
+    }
+  }
+  s1 = block_sum<256>(s1, red);
+  s2 = block_sum<256>(s2, red);
+  s3 = block_sum<256>(s3, red);
+  const float n = (float)F;
+  const float r1 = coef[0] / sqrtf(s1 / n + eps), r2 = coef[1] / sqrtf(s2 / n + eps),
+              r3 = coef[2] / sqrtf(s3 / n + eps), e = coef[3];
+#pragma unroll
+  for (int k = 0; k < NCH; ++k) {
+    const int c = threadIdx.x + k * 256;
+    if (c < nv) {
+      bf16x8 o;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float x = (float)v[k][j];
+        o[j] = (bf16)(x * (r1 + x * (r2 + x * r3)) + e);
+      }
+      *(bf16x8*)(out + row * out_stride + c * 8) = o;
+    }
+  }
+}
+
 OME_API int ome_polynorm(const void* z, int64_t z_stride, const float* coef, void* out, int64_t out_stride, int rows,
                          int F, float eps, int f32, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (F <= 0) return -2;
+  if (!f32 && F % 8 == 0 && F <= 8 * 256 * 16 && z_stride % 8 == 0 && out_stride % 8 == 0 && aligned16(z) &&
+      aligned16(out)) {
+    const int nch = (F / 8 + 255) / 256;
+#define PN_VEC(N) \
+  polynorm_vec_kernel<N><<<rows, 256, 0, stream>>>((const bf16*)z, z_stride, coef, (bf16*)out, out_stride, F, eps)
+    if (nch <= 1) PN_VEC(1);
+    else if (nch <= 2) PN_VEC(2);
+    else if (nch <= 4) PN_VEC(4);
+    else if (nch <= 8) PN_VEC(8);
+    else PN_VEC(16);
+#undef PN_VEC
+    OME_CHECK_LAUNCH();
+    return 0;
+  }
   if (f32)
     polynorm_kernel<float><<<rows, 256, 0, stream>>>((const float*)z, z_stride, coef, (float*)out, out_stride, F, eps);
   else

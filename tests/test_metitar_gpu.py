@@ -43,10 +43,13 @@ def _seqs(lens, slots, resets):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("T,H", [(1, 48), (37, 320), (5, 1030)])
-def test_post_norm_add_and_row_norm(T, H, dt):
+@pytest.mark.parametrize("T,H", [(1, 48), (37, 320), (5, 1030), (3, 4096), (2, 9000)])
+@pytest.mark.parametrize("view", [True, False])     # False: contiguous, 16-byte aligned rows (the vector kernels)
+def test_post_norm_add_and_row_norm(T, H, dt, view):
     torch.manual_seed(0)
     res, y = torch.randn(T, H) * 4, (torch.randn(T, H + 3) * 2 + 0.7).to(dt)[:, 3:]
+    if not view:
+        y = y.contiguous()
     w, b = (torch.rand(H) + 0.5).to(dt), (torch.randn(H) * 0.2).to(dt)
     for kind, bias in ((0, b), (1, None), (0, None)):
         r_ref = res.clone()
@@ -80,7 +83,8 @@ def test_conv_mix(C, K, lens, dt):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("H,d,vd,lens", [(6, 32, 32, [1, 9, 40]), (3, 48, 24, [17, 2]), (2, 128, 128, [20]),
-                                         (5, 16, 64, [1, 1]), (2, 3, 70, [11]), (1, 128, 256, [9, 1]), (4, 64, 5, [30])])
+                                         (5, 16, 64, [1, 1]), (2, 3, 70, [11]), (1, 128, 256, [9, 1]), (4, 64, 5, [30]), (1, 512, 64, [37]),
+                                         (2, 128, 128, [300]), (40, 16, 64, [1] * 3)])
 def test_hgrn2_scan(H, d, vd, lens, dt):
     torch.manual_seed(2)
     S = len(lens)
@@ -101,10 +105,11 @@ def test_hgrn2_scan(H, d, vd, lens, dt):
 def test_polynorm_gather_scale(dt):
     torch.manual_seed(3)
     coef = torch.tensor([0.9, -0.4, 0.3, 0.05])
-    for T, F in ((5, 320), (70, 13), (3, 1030)):
+    for T, F in ((5, 320), (70, 13), (3, 1030), (4, 14336), (2, 40000)):
         z = (torch.randn(T, F + 1) * 1.5).to(dt)[:, 1:]
-        assert _close(ops.polynorm(z.to(DEV), coef.to(DEV), 1e-6), ref.polynorm(z, coef, 1e-6, torch.empty(T, F, dtype=dt)),
-                      _tol(dt))
+        for zz in (z, z.contiguous()):      # a strided view, and aligned rows (the vector kernel)
+            assert _close(ops.polynorm(zz.to(DEV), coef.to(DEV), 1e-6),
+                          ref.polynorm(zz, coef, 1e-6, torch.empty(T, F, dtype=dt)), _tol(dt))
     g, ids, tab = torch.randn(9, 16).to(dt), torch.randint(0, 50, (9,), dtype=torch.int32), torch.randn(50, 96).to(dt)
     assert _close(ops.gelu_gather_mul(g.to(DEV), ids.to(DEV), tab.to(DEV), 32),
                   ref.gelu_gather_mul(g, ids, tab, 32, torch.empty_like(g)), _tol(dt))
