@@ -15,6 +15,7 @@
 namespace {
 
 constexpr int CH = 1024;
+constexpr int MAXD = 768;   // widest head (three output dims per thread)
 
 __device__ __forceinline__ float block_max256(float v, float* red) {
   v = wave_max(v);
@@ -31,7 +32,7 @@ __global__ __launch_bounds__(256) void paged_attention_f32_kernel(
     const float* __restrict__ v_cache, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ row_seq, const int* __restrict__ row_pos, float* __restrict__ out, int64_t out_stride,
     int Hq, int Hkv, int D, int P, float scale, int window, int keep, const float* __restrict__ sinks) {
-  __shared__ float qs[256];
+  __shared__ float qs[MAXD];
   __shared__ float sc[CH];
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
@@ -40,16 +41,16 @@ __global__ __launch_bounds__(256) void paged_attention_f32_kernel(
   const int pos = row_pos[t];
   float* orow = out + t * out_stride + (int64_t)h * D;
   if (pos < 0) {   // padding row: no keys
-    if (tid < D) orow[tid] = 0.f;
+    for (int d = tid; d < D; d += 256) orow[d] = 0.f;
     return;
   }
   const int* bt = block_tables + (int64_t)row_seq[t] * bt_stride;
   const int lo = window > 0 ? max(0, pos - window + 1) : (window < -1 ? pos - pos % (-window) : 0);
   const int kept = keep > 0 ? min(keep, lo) : 0;     // kept keys that lie before the window
   const int n_vis = kept + (pos - lo + 1);
-  if (tid < D) qs[tid] = q[t * q_stride + (int64_t)h * D + tid];
+  for (int d = tid; d < D; d += 256) qs[d] = q[t * q_stride + (int64_t)h * D + d];
   __syncthreads();
-  float m = -__builtin_inff(), l = 0.f, acc = 0.f;
+  float m = -__builtin_inff(), l = 0.f, acc[3] = {0.f, 0.f, 0.f};   // output dims tid, tid + 256, tid + 512
   for (int c0 = 0; c0 < n_vis; c0 += CH) {
     const int n = min(CH, n_vis - c0);
     float cm = -__builtin_inff();
@@ -74,11 +75,15 @@ __global__ __launch_bounds__(256) void paged_attention_f32_kernel(
     const float alpha = expf(m - m_new);  // first chunk: exp(-inf) = 0
     l = l * alpha + ps;
     m = m_new;
-    if (tid < D) {
-      acc *= alpha;
-      for (int i = 0; i < n; ++i) {
-        const int key = c0 + i < kept ? c0 + i : lo + (c0 + i - kept);
-        acc += sc[i] * v_cache[(((int64_t)bt[key / P] * Hkv + kvh) * D + tid) * P + key % P];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+      const int d = tid + 256 * j;
+      if (d < D) {
+        acc[j] *= alpha;
+        for (int i = 0; i < n; ++i) {
+          const int key = c0 + i < kept ? c0 + i : lo + (c0 + i - kept);
+          acc[j] += sc[i] * v_cache[(((int64_t)bt[key / P] * Hkv + kvh) * D + d) * P + key % P];
+        }
       }
     }
     __syncthreads();
@@ -86,9 +91,12 @@ __global__ __launch_bounds__(256) void paged_attention_f32_kernel(
   if (sinks != nullptr) {
     const float sk = sinks[h], m_new = fmaxf(m, sk), alpha = expf(m - m_new);
     l = l * alpha + expf(sk - m_new);
-    acc *= alpha;
+#pragma unroll
+    for (int j = 0; j < 3; ++j) acc[j] *= alpha;
   }
-  if (tid < D) orow[tid] = acc / l;
+#pragma unroll
+  for (int j = 0; j < 3; ++j)
+    if (tid + 256 * j < D) orow[tid + 256 * j] = acc[j] / l;
 }
 
 }  // namespace
@@ -98,7 +106,7 @@ OME_API int ome_paged_attention_f32(const float* q, int64_t q_stride, const floa
                                     float* out, int64_t out_stride, int T, int Hq, int Hkv, int D, int P, float scale,
                                     int window, int keep_first, const float* sinks, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (D <= 0 || D > 256 || P <= 0 || Hkv <= 0 || Hq % Hkv != 0) return -2;
+  if (D <= 0 || D > MAXD || P <= 0 || Hkv <= 0 || Hq % Hkv != 0) return -2;
   paged_attention_f32_kernel<<<dim3(T, Hq), 256, 0, stream>>>(q, q_stride, k_cache, v_cache, block_tables, bt_stride,
                                                               row_seq, row_pos, out, out_stride, Hq, Hkv, D, P, scale,
                                                               window, window > 0 && keep_first > 0 ? keep_first : 0,

@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void mla_attn_kernel(
     const bf16* __restrict__ q, int64_t q_stride_t, const bf16* __restrict__ cache,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tok_row,
     const int* __restrict__ kv_lens, int H, float scale_log2, int parts, bf16* __restrict__ out,
-    int64_t out_stride_t, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
+    int64_t out_stride_t, float* __restrict__ ws_o, float* __restrict__ ws_ml, const float* __restrict__ sinks) {
   constexpr int CH = DK / 8, NB = DV / 64, NST = (KT * CH + 255) / 256;   // NB 16-dim blocks per wave
   __shared__ __attribute__((aligned(16))) bf16 sK[KT * lds_chunks<DK>() * 8];
   const int t = blockIdx.x, h0 = blockIdx.y * 16, part = blockIdx.z;
@@ -164,6 +164,17 @@ __global__ __launch_bounds__(256) void mla_attn_kernel(
   }
 
   // ---- epilogue: O^T lane map dim = 16 nb + 4 g + i, head = col ----
+  // sinks (optional, fp32 [H], natural-log units, unscaled): exp(sink_h) joins head h's softmax
+  // denominator once, with no value; unsplit here, after the merge of the partials otherwise
+  if (sinks != nullptr && parts == 1 && hv) {
+    const float sk = sinks[h0 + col] * 1.4426950408889634f;
+    const float m_fin = fmaxf(m, sk), a = __builtin_amdgcn_exp2f(m - m_fin);
+    lsum = lsum * a + __builtin_amdgcn_exp2f(sk - m_fin);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[nb][i] *= a;
+  }
   const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
   if (!hv) return;
   if (parts == 1) {
@@ -352,7 +363,8 @@ __global__ __launch_bounds__(64 * NW, 1) void mla_attn_all_kernel(
 template <int DV>
 __global__ __launch_bounds__(128) void mla_reduce_kernel(const float* __restrict__ ws_o,
                                                          const float* __restrict__ ws_ml, int H, int parts,
-                                                         bf16* __restrict__ out, int64_t out_stride_t) {
+                                                         bf16* __restrict__ out, int64_t out_stride_t,
+                                                         const float* __restrict__ sinks) {
   const int t = blockIdx.x, h = blockIdx.y;
   const int64_t row0 = ((int64_t)t * H + h) * parts;
   float M = OME_NEG_INF, den = 0.f;
@@ -377,6 +389,12 @@ __global__ __launch_bounds__(128) void mla_reduce_kernel(const float* __restrict
       M = mn;
     }
   }
+  if (sinks != nullptr) {
+    const float sk = sinks[h] * 1.4426950408889634f;
+    const float mn = fmaxf(M, sk), a = __builtin_amdgcn_exp2f(M - mn);
+    acc = acc * a;
+    den = den * a + __builtin_amdgcn_exp2f(sk - mn);
+  }
   const float inv = den > 0.f ? 1.f / den : 0.f;
   bf16x4 r;
 #pragma unroll
@@ -391,7 +409,8 @@ __global__ __launch_bounds__(128) void mla_reduce_kernel(const float* __restrict
 template <int DK, int DV>
 static void mla_launch(const void* q, int64_t q_stride_t, const void* cache, const int* block_tables, int bt_stride,
                        const int* tok_row, const int* kv_lens, int T, int H, float scale_log2, int parts, void* out,
-                       int64_t out_stride_t, float* ws_o, float* ws_ml, hipStream_t stream) {
+                       int64_t out_stride_t, float* ws_o, float* ws_ml, hipStream_t stream,
+                       const float* sinks = nullptr) {
   // all-heads kernel when the heads tile into groups of 128 (DeepSeek-V3 / Kimi-K2 at TP 1) or 64
   // (TP 2): one latent stream per token and partition; else the 16-head kernel.  OME_MLA_ALL=0
   // forces the 16-head kernel (A/B timing).  Batches of at most OME_MLA_ALL_MIN_T tokens (default
@@ -403,7 +422,9 @@ static void mla_launch(const void* q, int64_t q_stride_t, const void* cache, con
   const bool all_ok = all_env && T > min_t;
   bool done = false;
   if constexpr (DK == 576) {
-    if (all_ok && H % 128 == 0) {
+    if (sinks != nullptr) {
+      // (the all-heads kernel has no sink term: sinks take the 16-head kernel)
+    } else if (all_ok && H % 128 == 0) {
       mla_attn_all_kernel<DK, DV, 8><<<dim3(T, H / 128, parts), 512, 0, stream>>>(
           (const bf16*)q, q_stride_t, (const bf16*)cache, block_tables, bt_stride, tok_row, kv_lens, H, scale_log2,
           parts, (bf16*)out, out_stride_t, ws_o, ws_ml);
@@ -418,9 +439,9 @@ static void mla_launch(const void* q, int64_t q_stride_t, const void* cache, con
   if (!done)
     mla_attn_kernel<DK, DV><<<dim3(T, (H + 15) / 16, parts), 256, 0, stream>>>(
         (const bf16*)q, q_stride_t, (const bf16*)cache, block_tables, bt_stride, tok_row, kv_lens, H, scale_log2,
-        parts, (bf16*)out, out_stride_t, ws_o, ws_ml);
+        parts, (bf16*)out, out_stride_t, ws_o, ws_ml, sinks);
   if (parts > 1)
-    mla_reduce_kernel<DV><<<dim3(T, H), DV / 4, 0, stream>>>(ws_o, ws_ml, H, parts, (bf16*)out, out_stride_t);
+    mla_reduce_kernel<DV><<<dim3(T, H), DV / 4, 0, stream>>>(ws_o, ws_ml, H, parts, (bf16*)out, out_stride_t, sinks);
 }
 
 OME_API int ome_mla_attn(const void* q, int64_t q_stride_t, const void* cache, const int* block_tables,
@@ -440,6 +461,39 @@ OME_API int ome_mla_attn(const void* q, int64_t q_stride_t, const void* cache, c
     return -3;
   OME_CHECK_LAUNCH();
   return 0;
+}
+
+// Latent attention over rows of any latent / rotary width, padded to the kernel's tiling: a cache
+// row is [latent (dv_pad wide: the values, zero beyond the latent) | rotary key (dk - dv_pad wide,
+// zero beyond it)], dv_pad a multiple of 64 up to 256 or 512, dk - dv_pad 32 or 64.  The 16-head kernel
+// serves every step kind; sinks optional.  Zero columns add nothing to a score, and the output's
+// zero columns are dropped by the caller.
+OME_API int ome_latent_attn(const void* q, int64_t q_stride_t, const void* cache, const int* block_tables,
+                            int bt_stride, const int* tok_row, const int* kv_lens, int T, int H, int dk, int dv,
+                            float scale, int parts, void* out, int64_t out_stride_t, float* ws_o, float* ws_ml,
+                            const float* sinks, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H <= 0 || parts < 1 || (parts > 1 && (!ws_o || !ws_ml))) return -2;
+  const float scale_log2 = scale * 1.4426950408889634f;
+#define LATENT_CASE(DK_, DV_)                                                                                       \
+  if (dk == DK_ && dv == DV_) {                                                                                     \
+    mla_launch<DK_, DV_>(q, q_stride_t, cache, block_tables, bt_stride, tok_row, kv_lens, T, H, scale_log2, parts,  \
+                         out, out_stride_t, ws_o, ws_ml, stream, sinks);                                            \
+    OME_CHECK_LAUNCH();                                                                                             \
+    return 0;                                                                                                       \
+  }
+  LATENT_CASE(96, 64)
+  LATENT_CASE(128, 64)
+  LATENT_CASE(160, 128)
+  LATENT_CASE(192, 128)
+  LATENT_CASE(224, 192)
+  LATENT_CASE(256, 192)
+  LATENT_CASE(288, 256)
+  LATENT_CASE(320, 256)
+  LATENT_CASE(544, 512)
+  LATENT_CASE(576, 512)
+#undef LATENT_CASE
+  return -3;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -510,24 +564,25 @@ OME_API int ome_mla_prep(const void* a, int64_t lda, int qlr, int lat, int rope,
 }
 
 // ------------------------------------------------------------------------------------------
-// Latent-attention glue for the generic paged attention kernels (any latent width / rotary width,
-// bf16 or fp32): the absorbed form is multi-query attention with ONE shared head whose key is
-// [RMSNorm(c) * w | rotated k_pe] and whose value is the latent RMSNorm(c) * w itself.  From the
-// fused down-projection output a [T, qlr + lat + rope] this writes, per token,
-//   K cache row   [page, 0, off, 0 : lat + rope]  (row-major keys, head width D >= lat + rope)
-//   V cache column [page, 0, 0 : lat, off]        (the value layout of the attention kernels)
-// (the tails up to D are never written: the caches start as zeros) and, for every head, the rotated
-// q_pe into qf[t, h, lat : lat + rope] with zeros up to D.  Rotary pairs are (j, j + rope/2), angles
-// from the fp32 table row of the token's position (cos | sin, any frequency scaling baked in).
-// k_cache == nullptr: a layer that reads another layer's cache only rotates its queries.
-// Padding rows (slot < 0) write slot 0 of the scratch page.
+// Latent-attention glue (any latent width / rotary width, bf16 or fp32): the absorbed form is
+// multi-query attention with ONE shared head whose key is [RMSNorm(c) * w | rotated k_pe] and whose
+// value is the latent RMSNorm(c) * w itself.  From the fused down-projection output a [T, qlr + lat
+// + rope] this writes, per token, the key row  k_cache[slot, 0 : lat] = latent,  k_cache[slot,
+// rope_off : rope_off + rope] = rotated k_pe  (rows D wide, rope_off >= lat; the gaps are never
+// written: the caches start as zeros) and -- only for the generic paged attention kernels, which
+// read values from their own array -- the value column v_cache[page, 0, 0 : lat, off]; the latent
+// kernel (ome_latent_attn) takes its values from the key rows, so v_cache is nullptr there.  For
+// every head the rotated q_pe goes to qf[t, h, rope_off : rope_off + rope], zeros into the gaps up
+// to D.  Rotary pairs are (j, j + rope/2), angles from the fp32 table row of the token's position
+// (cos | sin, any frequency scaling baked in).  k_cache == nullptr: a layer that reads another
+// layer's cache only rotates its queries.  Padding rows (slot < 0) write slot 0 of the scratch page.
 // ------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void latent_prep_kernel(
     const T* __restrict__ a, int64_t lda, int qlr, int lat, int rope, const T* __restrict__ w, float eps,
     const int* __restrict__ pos, const float* __restrict__ cs, const int* __restrict__ slots,
-    T* __restrict__ k_cache, T* __restrict__ v_cache, int D, int P, const T* __restrict__ q, int64_t q_tok,
-    int64_t q_head, int nope, int H, T* __restrict__ qf, int64_t qf_tok, int64_t qf_head) {
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int D, int P, int rope_off, const T* __restrict__ q,
+    int64_t q_tok, int64_t q_head, int nope, int H, T* __restrict__ qf, int64_t qf_tok, int64_t qf_head) {
   __shared__ float red[4];
   const int t = blockIdx.x, tid = threadIdx.x;
   const int half = rope >> 1;
@@ -537,7 +592,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
     int slot = slots[t];
     slot = slot < 0 ? 0 : slot;
     T* krow = k_cache + (int64_t)slot * D;
-    T* vcol = v_cache + (int64_t)(slot / P) * D * P + slot % P;
+    T* vcol = v_cache != nullptr ? v_cache + (int64_t)(slot / P) * D * P + slot % P : nullptr;
     float ss = 0.f;
     for (int i = tid; i < lat; i += 256) {
       const float v = (float)ar[i];
@@ -548,45 +603,46 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
     for (int i = tid; i < lat; i += 256) {
       const T v = (T)((float)ar[i] * rs * (float)w[i]);
       krow[i] = v;
-      vcol[(int64_t)i * P] = v;
+      if (vcol != nullptr) vcol[(int64_t)i * P] = v;
     }
     for (int j = tid; j < half; j += 256) {
       const float x1 = (float)ar[lat + j], x2 = (float)ar[lat + half + j];
       const float co = c[j], si = c[half + j];
-      krow[lat + j] = (T)(x1 * co - x2 * si);
-      krow[lat + half + j] = (T)(x2 * co + x1 * si);
+      krow[rope_off + j] = (T)(x1 * co - x2 * si);
+      krow[rope_off + half + j] = (T)(x2 * co + x1 * si);
     }
   }
-  const int tail = D - lat - rope;
+  const int gap = rope_off - lat, tail = D - rope_off - rope;
   for (int k = tid; k < H * half; k += 256) {
     const int h = k / half, j = k - h * half;
     const T* qr = q + (int64_t)t * q_tok + (int64_t)h * q_head + nope;
     const float x1 = (float)qr[j], x2 = (float)qr[half + j];
     const float co = c[j], si = c[half + j];
-    T* o = qf + (int64_t)t * qf_tok + (int64_t)h * qf_head + lat;
+    T* o = qf + (int64_t)t * qf_tok + (int64_t)h * qf_head + rope_off;
     o[j] = (T)(x1 * co - x2 * si);
     o[half + j] = (T)(x2 * co + x1 * si);
   }
-  for (int k = tid; k < H * tail; k += 256) {
-    const int h = k / tail, j = k - h * tail;
-    qf[(int64_t)t * qf_tok + (int64_t)h * qf_head + lat + rope + j] = (T)0.f;
+  for (int k = tid; k < H * (gap + tail); k += 256) {
+    const int h = k / (gap + tail), j = k - h * (gap + tail);
+    qf[(int64_t)t * qf_tok + (int64_t)h * qf_head + (j < gap ? lat + j : rope_off + rope + j - gap)] = (T)0.f;
   }
 }
 
 OME_API int ome_latent_prep(const void* a, int64_t lda, int qlr, int lat, int rope, const void* w, float eps,
                             const int* pos, const float* cs, const int* slots, void* k_cache, void* v_cache, int D,
-                            int P, const void* q, int64_t q_tok, int64_t q_head, int nope, int H, void* qf,
-                            int64_t qf_tok, int64_t qf_head, int T, int f32, hipStream_t stream) {
+                            int P, int rope_off, const void* q, int64_t q_tok, int64_t q_head, int nope, int H,
+                            void* qf, int64_t qf_tok, int64_t qf_head, int T, int f32, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (rope % 2 || lat <= 0 || H <= 0 || lat + rope > D || P <= 0) return -2;
+  if (rope % 2 || lat <= 0 || H <= 0 || rope_off < lat || rope_off + rope > D || P <= 0) return -2;
   if (f32)
     latent_prep_kernel<float><<<T, 256, 0, stream>>>((const float*)a, lda, qlr, lat, rope, (const float*)w, eps, pos,
-                                                     cs, slots, (float*)k_cache, (float*)v_cache, D, P,
+                                                     cs, slots, (float*)k_cache, (float*)v_cache, D, P, rope_off,
                                                      (const float*)q, q_tok, q_head, nope, H, (float*)qf, qf_tok,
                                                      qf_head);
   else
     latent_prep_kernel<bf16><<<T, 256, 0, stream>>>((const bf16*)a, lda, qlr, lat, rope, (const bf16*)w, eps, pos, cs,
-                                                    slots, (bf16*)k_cache, (bf16*)v_cache, D, P, (const bf16*)q,
-                                                    q_tok, q_head, nope, H, (bf16*)qf, qf_tok, qf_head);
+                                                    slots, (bf16*)k_cache, (bf16*)v_cache, D, P, rope_off,
+                                                    (const bf16*)q, q_tok, q_head, nope, H, (bf16*)qf, qf_tok,
+                                                    qf_head);
   return (int)hipGetLastError();
 }

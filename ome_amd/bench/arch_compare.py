@@ -304,7 +304,7 @@ def kernel_table_metitar(T: int = 4096, B: int = 64, ctx: int = 4096, width: int
         pair(f"polynorm ({tag})", lambda: ops.polynorm(z, coef, 1e-6), lambda: ops.act_and_mul(gu, 0), R * I * 4,
              R * I * 6, "two passes over the row (three mean squares, then the sum)")
         # ---- latent glue vs the MLA glue
-        qlr, lat, rope, D, P = 1536, 224, 32, 256, 16
+        qlr, lat, rope, D, P = 1536, 224, 32, 288, 16
         a = torch.randn(R, qlr + lat + rope, device=dev).to(bf)
         a2 = torch.randn(R, qlr + 256 + rope, device=dev).to(bf)
         nw, nw2 = torch.ones(lat, device=dev, dtype=bf), torch.ones(256, device=dev, dtype=bf)
@@ -313,15 +313,14 @@ def kernel_table_metitar(T: int = 4096, B: int = 64, ctx: int = 4096, width: int
         cs = yarn_rope_table(10000.0, rope, 2048, None, dev)
         q = torch.randn(R, H, 128 + rope, device=dev).to(bf)
         kc = torch.zeros(R // P + 2, 1, P, D, device=dev, dtype=bf)
-        vc = torch.zeros(R // P + 2, 1, D, P, device=dev, dtype=bf)
         qf = torch.empty(R, H, D, device=dev, dtype=bf)
         lc = torch.zeros((R // P + 2) * P, 288, device=dev, dtype=bf)
         qf2 = torch.empty(R, H, 288, device=dev, dtype=bf)
         nb = R * ((lat + rope) * 2 * 2 + H * rope * 2 * 2)
         pair(f"latent_prep ({tag})",
-             lambda: ops.latent_prep(a, qlr, lat, rope, nw, 1e-6, pos, cs, slots, kc, vc, q, 128, qf),
-             lambda: ops.mla_prep(a2, qlr, 256, rope, nw2, 1e-6, pos, cs, slots, lc, q, 128, qf2), nb + R * lat * 2, nb,
-             "writes the latent twice (key row, value column)")
+             lambda: ops.latent_prep(a, qlr, lat, rope, nw, 1e-6, pos, cs, slots, kc, None, q, 128, qf, rope_off=256),
+             lambda: ops.mla_prep(a2, qlr, 256, rope, nw2, 1e-6, pos, cs, slots, lc, q, 128, qf2), nb, nb,
+             "same glue with a rotary offset and zero fill of the row's gaps")
         # ---- routed feed-forward, router score on the expert's input vs on its output
         E, k, ff = 32, 4, 2048
         moe = InputScaledMoE(width, E, k, ff, 0, dev, bf)
@@ -333,43 +332,35 @@ def kernel_table_metitar(T: int = 4096, B: int = 64, ctx: int = 4096, width: int
         pair(f"input-scaled moe 32 experts top 4 ({tag})", lambda: moe.forward(x),
              lambda: ops.fused_moe(x, tw, tid, moe.w13, moe.w2, 0, 1.0), touched, touched,
              "new: router GEMM + route + row scaling + grouped GEMMs + unit-weight combine; like: grouped GEMMs + combine")
-    # ---- latent attention, decode: multi-query over 256-wide cache rows with sinks vs the MLA kernel
-    Hq, D, P = 16, 256, 16
+    # ---- latent attention: the 16-head MFMA latent kernel with sinks (288-wide rows: 224 latent + 32 rotary,
+    # padded) vs the same kernel as DeepSeek-style MLA runs it (no sinks)
+    Hq, DK, DV, P = 16, 288, 256, 16
     per = ctx // P
-    kc = (torch.randn(B * per + 1, 1, P, D, device=dev) * 0.3).to(bf)
-    vc = (torch.randn(B * per + 1, 1, D, P, device=dev) * 0.3).to(bf)
-    lc = (torch.randn(B * per + 1, P, 288, device=dev) * 0.3).to(bf)
+    lc = (torch.randn(B * per + 1, P, DK, device=dev) * 0.3).to(bf)
     bt = (torch.arange(B * per, dtype=torch.int32, device=dev) + 1).view(B, per)
     sl = torch.full((B,), ctx, dtype=torch.int32, device=dev)
-    q = torch.randn(B, Hq, D, device=dev).to(bf)
-    q2 = torch.randn(B, Hq, 288, device=dev).to(bf)
+    q2 = torch.randn(B, Hq, DK, device=dev).to(bf)
     sinks = torch.zeros(Hq, device=dev)
-    ws = ops.DecodeWorkspace(B, Hq, D, ctx, 0, dev, parts=16)
     mws = ops.MLAWorkspace(dev)
     rows_i = torch.arange(B, dtype=torch.int32, device=dev)
     pair("latent attention decode 64 x 4096 ctx, 16 heads",
-         lambda: ops.paged_decode(q, kc, vc, bt, sl, 0.08, ws, sinks=sinks),
-         lambda: ops.mla_attn(q2, lc, bt, rows_i, sl, 0.08, mws, dv=256), B * ctx * 256 * 2, B * ctx * 288 * 2,
-         "bytes that must move = the latent once; this path reads it as key and again as value")
+         lambda: ops.latent_attn(q2, lc, bt, rows_i, sl, 0.08, DV, mws, sinks=sinks),
+         lambda: ops.mla_attn(q2, lc, bt, rows_i, sl, 0.08, mws, dv=DV), B * ctx * DK * 2, B * ctx * DK * 2,
+         "the latent row is read once, for keys and values")
     # ---- latent attention, prefill 2 x 2048 rows
     q_lens = [2048, 2048]
     Tq = sum(q_lens)
-    qp = torch.randn(Tq, Hq, D, device=dev).to(bf)
-    qp2 = torch.randn(Tq, Hq, 288, device=dev).to(bf)
-    cu = torch.tensor([0, 2048, 4096], dtype=torch.int32, device=dev)
-    kl = torch.tensor(q_lens, dtype=torch.int32, device=dev)
+    qp2 = torch.randn(Tq, Hq, DK, device=dev).to(bf)
     bt2 = (torch.arange(2 * 128, dtype=torch.int32, device=dev) + 1).view(2, 128)
-    items = torch.tensor(ops.prefill_work_items(q_lens, q_lens), dtype=torch.int32, device=dev)
     tok_row = torch.arange(Tq, dtype=torch.int32, device=dev) // 2048
     tok_len = (torch.arange(Tq, dtype=torch.int32, device=dev) % 2048 + 1).to(torch.int32)
-    fl_new = 2.0 * Hq * (256 + 256) * sum(i + 1 for i in range(2048)) * 2
-    fl_like = 2.0 * Hq * (288 + 256) * sum(i + 1 for i in range(2048)) * 2
-    tn = _time_us(lambda: ops.paged_prefill(qp, kc, vc, bt2, cu, kl, items, 0.08, sinks=sinks), 10)
-    tl = _time_us(lambda: ops.mla_attn(qp2, lc, bt2, tok_row, tok_len, 0.08, mws, dv=256), 10)
-    rn, rl = fl_new / tn / 1e6 / 2.5e3, fl_like / tl / 1e6 / 2.5e3
+    fl = 2.0 * Hq * (DK + DV) * sum(i + 1 for i in range(2048)) * 2
+    tn = _time_us(lambda: ops.latent_attn(qp2, lc, bt2, tok_row, tok_len, 0.08, DV, mws, sinks=sinks), 10)
+    tl = _time_us(lambda: ops.mla_attn(qp2, lc, bt2, tok_row, tok_len, 0.08, mws, dv=DV), 10)
+    rn, rl = fl / tn / 1e6 / 2.5e3, fl / tl / 1e6 / 2.5e3
     rows.append({"kernel": "latent attention prefill 2 x 2048 rows, 16 heads", "us": round(tn, 1), "roofline": round(rn, 3),
                  "like_us": round(tl, 1), "like_roofline": round(rl, 3), "vs_like": round(rl / max(rn, 1e-9), 2),
-                 "note": "share of 2.5 PFLOP/s bf16; like: the MLA kernel on 288-wide rows"})
+                 "note": "share of 2.5 PFLOP/s bf16; one token x 16 heads per work item"})
     return rows
 
 

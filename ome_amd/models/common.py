@@ -86,7 +86,7 @@ class PagedKVCache:
         own = set(self.local_layers)
         hk = (lambda i: per[i]) if per else (lambda i: num_kv_heads)  # noqa: E731
         hd = (lambda i: per_d[i]) if per_d else (lambda i: head_dim)  # noqa: E731
-        vd = (lambda i: per_d[i]) if per_d else (lambda i: self.v_dim)  # noqa: E731
+        vd = (lambda i: per_d[i]) if per_d and v_dim is None else (lambda i: self.v_dim)  # noqa: E731
         self.k = [torch.zeros(num_pages, hk(i), page_size, hd(i), dtype=dtype, device=device)
                   if i in own else None for i in range(num_layers)]
         self.v = [torch.zeros(num_pages, hk(i), vd(i), page_size, dtype=dtype, device=device)
@@ -111,9 +111,9 @@ class PagedKVCache:
     def bytes_per_page(num_layers: int, num_kv_heads: int, head_dim: int, page_size: int, dtype=torch.bfloat16,
                        v_dim: int | None = None) -> int:
         esz = torch.tensor([], dtype=dtype).element_size()
-        if isinstance(head_dim, dict):   # per-layer widths (keys and values equally wide)
+        if isinstance(head_dim, dict):   # per-layer widths (values as wide as the keys, or ``v_dim`` for all)
             hk = num_kv_heads if isinstance(num_kv_heads, dict) else {i: num_kv_heads for i in head_dim}
-            return sum(hk[i] * 2 * d for i, d in head_dim.items()) * page_size * esz
+            return sum(hk[i] * (d + (d if v_dim is None else v_dim)) for i, d in head_dim.items()) * page_size * esz
         v = head_dim if v_dim is None else v_dim
         heads = sum(num_kv_heads.values()) if isinstance(num_kv_heads, dict) else num_layers * num_kv_heads
         return heads * (head_dim + v) * page_size * esz

@@ -140,6 +140,18 @@ def attn_tile_dim(d: int) -> int:
     raise ValueError(f"attention head width {d} exceeds the 256-wide kernel tile")
 
 
+def latent_row_width(kv_rank: int, rot_dim: int) -> int:
+    """Head width of the generic paged attention kernels for an absorbed latent-attention layer (one
+    shared head of latent + rotary key): the 64 / 128 / 256 tile, beyond it (fp32 models only: the
+    exact kernel takes any width up to 768) the next multiple of 64."""
+    d = kv_rank + rot_dim
+    if d <= 256:
+        return attn_tile_dim(d)
+    if d > 768:
+        raise ValueError(f"latent attention: latent + rotary width {d} exceeds 768")
+    return -(-d // 64) * 64
+
+
 def _layer_list_keys(c: dict[str, Any]) -> dict[str, Any]:
     """Layer-list configs (``architecture: Zavilorn`` / ``Metitar``): ``layers`` is a list of blocks,
     each with its mixer ``type``, the mixer's own sizes and its feed-forward.  The standard keys
@@ -153,7 +165,7 @@ def _layer_list_keys(c: dict[str, Any]) -> dict[str, Any]:
             dims.append(attn_tile_dim(max(m["left"]["dim"], m["left"]["vdim"])))
         elif L.get("type") == "latent_attention":   # absorbed form: one shared head of latent + rotary width
             attn.append(m)
-            dims.append(attn_tile_dim(m["kv_rank"] + m["rot_dim"]))
+            dims.append(latent_row_width(m["kv_rank"], m["rot_dim"]))
     ff = [(L["mlp"].get("ff") or (L["mlp"].get("expert") or {}).get("ff") or 0) for L in c["layers"] if L.get("mlp")]
     D = max(dims or [64])
     out = dict(c)

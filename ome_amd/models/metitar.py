@@ -25,7 +25,9 @@ norm, rotary angles, router logits, gates, the recurrence and its state are fp32
 kernels; logits leave the head in fp32.
 
 Cache and state: latent-attention layers that own a key/value projection own KV pages
-(``kv_layers``; one shared head of width tile(kv_rank + rot_dim) per layer); per request slot every
+(``kv_layers``; one shared row per token: in bf16 ``[latent | rotary key]`` padded to a shape of the
+latent kernel, values read from the same row; in fp32 key rows + value columns of the generic
+kernels); per request slot every
 layer keeps its conv tail and every HGRN2 layer its fp32 state (``alloc_state``).  Prefix caching
 is off (``stateful``).  The model has no cache, loop or scheduler of its own: ``ModelRunner``
 drives it like the other hybrids.
@@ -67,6 +69,10 @@ class MetitarForCausalLM(LlamaForCausalLM):
         self.rec: dict[int, Hgrn2Mixer] = {}
         self.ff: dict[int, PolyNormMLP | InputScaledMoE] = {}
         self.side: dict[int, TokenSideInput] = {}
+        lat = [s["mixer"] for s in self.specs if s["type"] == "latent_attention"]
+        # one cache layout for all attention layers: key rows that carry their values (the latent kernel,
+        # bf16) when every layer's widths have a kernel shape, else key rows + value columns
+        self.latent_cache = dtype == torch.bfloat16 and all(ops.latent_shape(m["kv_rank"], m["rot_dim"]) for m in lat)
         for i, spec in enumerate(self.specs):
             m = spec["mixer"]
             if spec["type"] == "latent_attention":
@@ -82,7 +88,7 @@ class MetitarForCausalLM(LlamaForCausalLM):
                     raise ValueError(f"layer {i}: rot.dims {rot.get('dims')} != rot_dim {m['rot_dim']}")
                 self.attn[i] = LatentAttention(i, src, W, m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"],
                                                m["q_rank"], rot["base"], rot.get("scaling"), m["scale"], eps, mp,
-                                               self.device, dtype)
+                                               self.device, dtype, self.latent_cache)
             elif spec["type"] == "hgrn2":
                 self.rec[i] = Hgrn2Mixer(W, m["heads"], m["dim"], m["vdim"], eps, self.device, dtype)
             else:
@@ -107,6 +113,7 @@ class MetitarForCausalLM(LlamaForCausalLM):
         self.kv_layers = sorted(i for i, a in self.attn.items() if a.own_cache)
         self.kv_heads_per_layer = {i: 1 for i in self.kv_layers}
         self.kv_dims_per_layer = {i: self.attn[i].D for i in self.kv_layers}
+        self.kv_value_dim = 0 if self.latent_cache else None      # (0: no value array beside the key rows)
         self.debug_residuals: list | None = None   # set to []: the residual after every layer is appended
 
     def prefill_item_rows(self, page: int) -> int:

@@ -34,7 +34,7 @@ import torch
 
 from ome_amd import ops
 from ome_amd.models.common import AttnMeta, PagedKVCache, mixed_attention
-from ome_amd.models.config import attn_tile_dim, plain_rope_table, yarn_rope_table
+from ome_amd.models.config import attn_tile_dim, latent_row_width, plain_rope_table, yarn_rope_table
 from ome_amd.models.quant import linear
 
 
@@ -261,16 +261,24 @@ class LatentAttention(_Block):
     pairs are (i, i + rot_dim/2) with the YaRN-scaled table of ``config.yarn_rope_table``.
 
     Runs absorbed: q_lat = W_uk^T q_nope, so all heads share one key [c | rope(k_pe)] and one value
-    c per token -- multi-query attention over a paged cache of head width D = tile(kv_rank +
-    rot_dim) (``ops.latent_prep`` -> ``paged_attention`` -> W_uv per head).  ``kv_layer`` != ``layer``:
-    this layer has no W_dkv and attends over ``kv_layer``'s cache rows with its own W_uk / W_uv.
-    Checkpoint tensors ``dq dq.norm uq [dkv dkv.norm] uk uv sink o``."""
+    c per token -- multi-query attention over one cached row per token, whatever the head count.
+    Two cache layouts (``latent_cache``, chosen by the model for all its layers):
 
-    HEAD_GROUP = 16   # query heads per kv head one attention launch takes
+    * key rows that carry their own values, ``[c | 0 .. | rope(k_pe) | 0 ..]`` in one of the widths of
+      ``ops.LATENT_SHAPES`` (bf16): ``ops.latent_prep`` -> ``ops.latent_attn`` (the 16-head MFMA latent
+      kernel: one launch for prompt chunks, decode rows and mixed batches) -> W_uv per head;
+    * key rows + value columns of the generic paged attention kernels, head width
+      ``config.latent_row_width`` (fp32 models, and widths the latent kernel is not built for):
+      ``ops.latent_prep`` -> ``paged_attention`` (more than 16 heads in groups of 16) -> W_uv.
+
+    ``kv_layer`` != ``layer``: this layer has no W_dkv and attends over ``kv_layer``'s cache rows with
+    its own W_uk / W_uv.  Checkpoint tensors ``dq dq.norm uq [dkv dkv.norm] uk uv sink o``."""
+
+    HEAD_GROUP = 16   # query heads per kv head one launch of the generic attention kernels takes
 
     def __init__(self, layer: int, kv_layer: int, width: int, heads: int, dim: int, rot_dim: int, vdim: int,
                  kv_rank: int, q_rank: int, rot_base: float, rot_scaling: dict | None, scale: float, eps: float,
-                 max_positions: int, device, dtype):
+                 max_positions: int, device, dtype, latent_cache: bool | None = None):
         super().__init__(device, dtype)
         if rot_dim % 2 or rot_dim <= 0:
             raise ValueError(f"latent attention: rotary width {rot_dim} must be even and positive")
@@ -278,7 +286,15 @@ class LatentAttention(_Block):
         self.dim, self.rot, self.vdim, self.R, self.qr = dim, rot_dim, vdim, kv_rank, q_rank
         self.scale, self.eps = float(scale), float(eps)
         self.own_cache = kv_layer == layer
-        self.D = attn_tile_dim(kv_rank + rot_dim)
+        shape = ops.latent_shape(kv_rank, rot_dim) if dtype == torch.bfloat16 else None
+        self.latent_cache = shape is not None if latent_cache is None else bool(latent_cache)
+        if self.latent_cache:
+            if shape is None:
+                raise ValueError(f"latent attention: no latent kernel for a {kv_rank} + {rot_dim}-wide row in {dtype}")
+            self.D, self.DV = shape              # row width, value width (= where the rotary key starts)
+        else:
+            self.D = latent_row_width(kv_rank, rot_dim)
+            self.DV = kv_rank
         self.cos_sin = yarn_rope_table(rot_base, rot_dim, max_positions, rot_scaling, self.device)
         self.w_in = self.qn = self.w_uq = self.kvn = self.w_uk = self.w_uv = self.sink = self.w_o = None
 
@@ -307,21 +323,67 @@ class LatentAttention(_Block):
         T, H, R, D = h.shape[0], self.H, self.R, self.D
         a = linear(h, self.w_in)                                          # [T, q_rank (| latent | k_pe)]
         q = linear(ops.row_norm(a[:, :self.qr], self.qn, None, self.eps, 1), self.w_uq).view(T, H, self.dim + self.rot)
-        q_full = torch.empty(T, H, D, dtype=h.dtype, device=h.device)     # [W_uk^T q_nope | rope(q_pe) | 0]
+        q_full = torch.empty(T, H, D, dtype=h.dtype, device=h.device)     # [W_uk^T q_nope | 0 | rope(q_pe) | 0]
         k_cache, v_cache = ctx.kv.layer(self.kv_layer)
         own = self.own_cache
         ops.latent_prep(a, self.qr, R, self.rot, self.kvn, self.eps, ctx.meta.positions, self.cos_sin, ctx.meta.slots,
-                        k_cache if own else None, v_cache if own else None, q, self.dim, q_full)
+                        k_cache if own else None, v_cache if own and not self.latent_cache else None, q, self.dim,
+                        q_full, rope_off=self.DV)
         torch.bmm(q[..., :self.dim].transpose(0, 1), self.w_uk, out=q_full[:, :, :R].transpose(0, 1))
-        G = self.HEAD_GROUP
-        if H <= G:
-            o_lat = paged_attention(q_full, k_cache, v_cache, ctx.meta, self.scale, sinks=self.sink)
-        else:   # the kernels share one kv head among at most G query heads: run the heads in groups
-            o_lat = torch.cat([paged_attention(q_full[:, g:g + G], k_cache, v_cache, ctx.meta, self.scale,
-                                               sinks=self.sink[g:g + G]) for g in range(0, H, G)], 1)
+        if self.latent_cache:
+            o_lat = torch.empty(T, H, self.DV, dtype=h.dtype, device=h.device)
+            rows3 = k_cache.view(k_cache.shape[0], k_cache.shape[2], D)
+            ws = _latent_workspace(h)
+            for s, e, bt, rows, lens in latent_rows(ctx.meta, T):
+                ops.latent_attn(q_full[s:e], rows3, bt, rows, lens, self.scale, self.DV, ws, out=o_lat[s:e],
+                                sinks=self.sink)
+        else:
+            G = self.HEAD_GROUP
+            if H <= G:
+                o_lat = paged_attention(q_full, k_cache, v_cache, ctx.meta, self.scale, sinks=self.sink)
+            else:   # the kernels share one kv head among at most G query heads: run the heads in groups
+                o_lat = torch.cat([paged_attention(q_full[:, g:g + G], k_cache, v_cache, ctx.meta, self.scale,
+                                                   sinks=self.sink[g:g + G]) for g in range(0, H, G)], 1)
         o = torch.empty(T, H * self.vdim, dtype=h.dtype, device=h.device)
         torch.bmm(o_lat[:, :, :R].transpose(0, 1), self.w_uv, out=o.view(T, H, self.vdim).transpose(0, 1))
         return linear(o, self.w_o)
+
+
+_ARANGE: dict = {}
+_LATENT_WS: dict = {}
+
+
+def latent_rows(meta: AttnMeta, T: int) -> list:
+    """The step's rows as the latent attention kernel takes them: segments (first row, end row,
+    block table, block-table row per token, visible keys per token) -- one for the prompt chunks,
+    one for the single decode rows of a mixed step."""
+    dev = meta.positions.device
+    ar = _ARANGE.get(dev)
+    if ar is None or ar.numel() < T:
+        ar = _ARANGE[dev] = torch.arange(max(T, 4096), dtype=torch.int32, device=dev)
+    if meta.is_decode:
+        return [(0, T, meta.block_tables, ar[:T], meta.seq_lens)]
+    kv_lens = (meta.positions + 1).to(torch.int32)
+    n = meta.num_prefill if meta.mode == "mixed" else T
+    seg = []
+    if n:
+        cu = meta.cu_q
+        rows = torch.searchsorted(cu[1:].contiguous(), ar[:n].to(cu.dtype), right=True).to(torch.int32)
+        seg.append((0, n, meta.block_tables, rows, kv_lens[:n]))
+    if n < T:
+        seg.append((n, T, meta.dec_block_tables, ar[:T - n], meta.seq_lens))
+    return seg
+
+
+def _latent_workspace(x: torch.Tensor):
+    """Split-K partials of the latent kernel, one per stream (layers of a stream run in turn)."""
+    if not x.is_cuda:
+        return None
+    key = (x.device, torch.cuda.current_stream(x.device).cuda_stream)
+    ws = _LATENT_WS.get(key)
+    if ws is None:
+        ws = _LATENT_WS[key] = ops.MLAWorkspace(x.device)
+    return ws
 
 
 class Hgrn2Mixer(_Block):

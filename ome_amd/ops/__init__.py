@@ -1734,29 +1734,82 @@ def conv_mix(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor, cu, slot, re
 
 def latent_prep(a: torch.Tensor, qlr: int, lat: int, rope: int, w: torch.Tensor | None, eps: float,
                 positions: torch.Tensor, cos_sin: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor | None,
-                v_cache: torch.Tensor | None, q: torch.Tensor, nope: int, q_full: torch.Tensor) -> None:
-    """Latent attention before the paged attention kernels, in its absorbed (multi-query) form:
-    from the fused down projection ``a`` [T, qlr + lat + rope] write the token's key
-    ``[RMSNorm(c) * w | RoPE(k_pe)]`` into ``k_cache`` [pages, 1, P, D] and its value
-    ``RMSNorm(c) * w`` into ``v_cache`` [pages, 1, D, P] (D >= lat + rope; the tails stay zero),
-    and the rotated q_pe of every head into ``q_full[:, :, lat:lat + rope]`` (zeros up to D);
-    q [T, H, nope + rope].  Rotary pairs are (j, j + rope/2); ``cos_sin`` fp32 [positions, rope] =
-    cos | sin.  ``k_cache`` None: only the queries (a layer that reads another layer's cache)."""
+                v_cache: torch.Tensor | None, q: torch.Tensor, nope: int, q_full: torch.Tensor,
+                rope_off: int | None = None) -> None:
+    """Latent attention before the attention kernels, in its absorbed (multi-query) form: from the
+    fused down projection ``a`` [T, qlr + lat + rope] write the token's key row into ``k_cache``
+    [pages, 1, P, D]: ``RMSNorm(c) * w`` at columns [0, lat), ``RoPE(k_pe)`` at [rope_off, rope_off
+    + rope) (default ``rope_off = lat``; the gaps stay zero); with ``v_cache`` [pages, 1, D, P] (the
+    generic paged attention kernels) also the value column ``RMSNorm(c) * w``; and the rotated q_pe
+    of every head into ``q_full[:, :, rope_off:rope_off + rope]`` (zeros in the gaps up to D); q [T,
+    H, nope + rope].  Rotary pairs are (j, j + rope/2); ``cos_sin`` fp32 [positions, rope] = cos |
+    sin.  ``k_cache`` None: only the queries (a layer that reads another layer's cache)."""
+    rope_off = lat if rope_off is None else int(rope_off)
     if not _gpu(q):
-        return ref.latent_prep(a, qlr, lat, rope, w, eps, positions, cos_sin, slots, k_cache, v_cache, q, nope, q_full)
+        return ref.latent_prep(a, qlr, lat, rope, w, eps, positions, cos_sin, slots, k_cache, v_cache, q, nope, q_full,
+                               rope_off)
     T, H = q.shape[0], q.shape[1]
     D = q_full.shape[2]
+    assert lat <= rope_off and rope_off + rope <= D
     P = 1
     if k_cache is not None:
         P = k_cache.shape[2]
-        assert k_cache.shape[1] == 1 and k_cache.shape[3] == D and v_cache.shape[1:] == (1, D, P)
-        assert k_cache.is_contiguous() and v_cache.is_contiguous() and a.stride(1) == 1
+        assert k_cache.shape[1] == 1 and k_cache.shape[3] == D and k_cache.is_contiguous() and a.stride(1) == 1
+        assert v_cache is None or (v_cache.shape[1:] == (1, D, P) and v_cache.is_contiguous())
     f32 = _f32(q, q_full, k_cache, v_cache, w, a if k_cache is not None else None)
     assert q.stride(2) == 1 and q_full.stride(2) == 1
     assert cos_sin.dtype == torch.float32 and cos_sin.shape[1] == rope and cos_sin.is_contiguous()
     call("ome_latent_prep", a.data_ptr(), a.stride(0), qlr, lat, rope, ptr(w), float(eps), _i32(positions).data_ptr(),
-         cos_sin.data_ptr(), _i32(slots).data_ptr(), ptr(k_cache), ptr(v_cache), D, P, q.data_ptr(), q.stride(0),
-         q.stride(1), nope, H, q_full.data_ptr(), q_full.stride(0), q_full.stride(1), T, f32, stream_ptr())
+         cos_sin.data_ptr(), _i32(slots).data_ptr(), ptr(k_cache), ptr(v_cache), D, P, rope_off, q.data_ptr(),
+         q.stride(0), q.stride(1), nope, H, q_full.data_ptr(), q_full.stride(0), q_full.stride(1), T, f32,
+         stream_ptr())
+
+
+#: (row width, value width) pairs the latent attention kernel is built for: the value part a
+#: multiple of 64 (the latent, zero-padded), then 32 or 64 columns for the rotary key
+LATENT_SHAPES = ((96, 64), (128, 64), (160, 128), (192, 128), (224, 192), (256, 192), (288, 256), (320, 256),
+                 (544, 512), (576, 512))
+
+
+def latent_shape(lat: int, rope: int) -> tuple[int, int] | None:
+    """Smallest kernel shape (row width, value width) holding a ``lat``-wide latent and a
+    ``rope``-wide rotary key, or None when there is none."""
+    for dk, dv in LATENT_SHAPES:
+        if lat <= dv and rope <= dk - dv:
+            return dk, dv
+    return None
+
+
+def latent_attn(q, cache, block_tables, tok_row, kv_lens, scale: float, dv: int, ws: MLAWorkspace | None = None,
+                out: torch.Tensor | None = None, sinks: torch.Tensor | None = None) -> torch.Tensor:
+    """Absorbed latent attention over a paged cache of key rows that carry their own values: q [T,
+    H, DK], cache [pages, 16, DK] -> out [T, H, dv] (values = the first ``dv`` columns of a row);
+    (DK, dv) one of :data:`LATENT_SHAPES`.  Token t sees keys [0, kv_lens[t]) of block-table row
+    tok_row[t] (prompt chunks, decode rows and mixed batches alike).  ``sinks``: fp32 [H] logits
+    that join each head's softmax denominator (no key, no value, unscaled)."""
+    if not _gpu(q):
+        r = ref.mla_attn(q, cache, block_tables, tok_row, kv_lens, scale, dv, sinks)
+        if out is not None:
+            out.copy_(r)
+            return out
+        return r
+    T, H, DK = q.shape
+    assert (DK, dv) in LATENT_SHAPES, (DK, dv)
+    assert q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and cache.is_contiguous()
+    assert q.stride(2) == 1 and q.stride(1) == DK and cache.shape[-1] == DK and cache.shape[-2] == 16
+    if out is None:
+        out = torch.empty(T, H, dv, dtype=q.dtype, device=q.device)
+    assert out.stride(2) == 1 and out.stride(1) == dv
+    parts = MLAWorkspace.parts(T, H, DK)
+    if sinks is not None and DK == 576:   # (sinks run the 16-head kernel: partition as it does)
+        parts = MLAWorkspace.parts(T, H, 0)
+    if parts > 1 and ws is None:
+        ws = MLAWorkspace(q.device)
+    call("ome_latent_attn", q.data_ptr(), q.stride(0), cache.data_ptr(), _i32(block_tables).data_ptr(),
+         block_tables.stride(0), _i32(tok_row).data_ptr(), _i32(kv_lens).data_ptr(), T, H, DK, dv, float(scale),
+         parts, out.data_ptr(), out.stride(0), ws.ws_o.data_ptr() if parts > 1 else None,
+         ws.ws_ml.data_ptr() if parts > 1 else None, _sinks(sinks), stream_ptr())
+    return out
 
 
 def hgrn2_scan(q: torch.Tensor, f: torch.Tensor, v: torch.Tensor, f_bias: torch.Tensor, lower: torch.Tensor,

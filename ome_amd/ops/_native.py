@@ -51,8 +51,9 @@ _SIGNATURES = {
         "ome_gelu_gather_mul": [vp, i64, vp, vp, i64, i32, i32, vp, i32, i32, i32, vp],
         "ome_scale_rows": [vp, i64, vp, i32, vp, i32, i32, i32, vp],
         "ome_conv_mix": [vp, i64, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
-        "ome_latent_prep": [vp, i64, i32, i32, i32, vp, f32, vp, vp, vp, vp, vp, i32, i32, vp, i64, i64, i32, i32, vp,
-                            i64, i64, i32, i32, vp],
+        "ome_latent_prep": [vp, i64, i32, i32, i32, vp, f32, vp, vp, vp, vp, vp, i32, i32, i32, vp, i64, i64, i32, i32,
+                            vp, i64, i64, i32, i32, vp],
+        "ome_latent_attn": [vp, i64, vp, vp, i32, vp, vp, i32, i32, i32, i32, f32, i32, vp, i64, vp, vp, vp, vp],
         "ome_hgrn2_scan": [vp, vp, vp, i64, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, f32, i32, vp],
         "ome_act": [vp, i64, i32, vp],
         "ome_ssm_conv1d": [vp, i64, vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, vp],

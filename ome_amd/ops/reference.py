@@ -638,9 +638,9 @@ def fp8_gemm(qa, sa, qw, sw, block: int, bias=None, out_dtype=torch.bfloat16):
     return out.to(out_dtype)
 
 
-def mla_attn(q, cache, block_tables, tok_row, kv_lens, scale, dv=512):
+def mla_attn(q, cache, block_tables, tok_row, kv_lens, scale, dv=512, sinks=None):
     """Absorbed MLA: q [T, H, DK], cache [pages, 16, DK] -> out [T, H, dv] (values = the first dv
-    latent dims)."""
+    latent dims).  ``sinks``: fp32 [H] logits joining each head's softmax denominator."""
     T, H, DK = q.shape
     P = cache.shape[-2]
     out = torch.empty(T, H, dv, dtype=q.dtype, device=q.device)
@@ -650,7 +650,8 @@ def mla_attn(q, cache, block_tables, tok_row, kv_lens, scale, dv=512):
         pages = block_tables[int(tok_row[t])][: -(-L // P)].long()
         kv = flat[pages].reshape(-1, DK)[:L].float()
         s = (q[t].float() @ kv.t()) * scale
-        out[t] = (torch.softmax(s, -1) @ kv[:, :dv]).to(q.dtype)
+        sk = None if sinks is None else sinks.float().view(H, 1)
+        out[t] = (_softmax_sink(s, sk) @ kv[:, :dv]).to(q.dtype)
     return out
 
 
@@ -687,7 +688,7 @@ def conv_mix(x, w, state, cu, slot, reset, out):
     return out
 
 
-def latent_prep(a, qlr, lat, rope, w, eps, positions, cos_sin, slots, k_cache, v_cache, q, nope, q_full):
+def latent_prep(a, qlr, lat, rope, w, eps, positions, cos_sin, slots, k_cache, v_cache, q, nope, q_full, rope_off):
     cs = cos_sin.index_select(0, positions.long())
     half = rope // 2
 
@@ -701,10 +702,13 @@ def latent_prep(a, qlr, lat, rope, w, eps, positions, cos_sin, slots, k_cache, v
         cf = ckv[:, :lat].float()
         c = (cf * torch.rsqrt(cf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(a.dtype)
         sl = slots.long().clamp_min(0)
-        k_cache.view(-1, D)[sl, :lat + rope] = torch.cat([c, rot(ckv[:, lat:], cs[:, :half], cs[:, half:])], -1)
-        v_cache[sl // P, 0, :lat, sl % P] = c
-    q_full[:, :, lat:lat + rope] = rot(q[..., nope:], cs[:, None, :half], cs[:, None, half:])
-    q_full[:, :, lat + rope:] = 0
+        rows = k_cache.view(-1, D)
+        rows[sl, :lat] = c
+        rows[sl, rope_off:rope_off + rope] = rot(ckv[:, lat:], cs[:, :half], cs[:, half:])
+        if v_cache is not None:
+            v_cache[sl // P, 0, :lat, sl % P] = c
+    q_full[:, :, lat:] = 0
+    q_full[:, :, rope_off:rope_off + rope] = rot(q[..., nope:], cs[:, None, :half], cs[:, None, half:])
 
 
 def hgrn2_scan(q, f, v, f_bias, lower, w, state, cu, slot, reset, H, dim, vdim, eps, out):

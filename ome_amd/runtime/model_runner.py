@@ -190,7 +190,8 @@ class ModelRunner:
         if getattr(self.model, "kv_heads_per_layer", None):   # per-layer GQA (DeciLM): {layer: local heads}
             kv_heads = dict(self.model.kv_heads_per_layer)
         if getattr(self.model, "kv_dims_per_layer", None):    # per-layer head widths: {layer: D}
-            k_dim, v_dim = dict(self.model.kv_dims_per_layer), None
+            # (``kv_value_dim`` = 0: key rows that carry their own values, no value array)
+            k_dim, v_dim = dict(self.model.kv_dims_per_layer), getattr(self.model, "kv_value_dim", None)
         kv_dtype = kv_cache_dtype(kv_cache_dtype_name, dtype)
         if kv_dtype != dtype and getattr(self.model, "kv_layout", None) is not None:
             # MLA's latent cache (mla.hip) keeps the model dtype

@@ -118,9 +118,12 @@ def test_polynorm_gather_scale(dt):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("H,qlr,lat,rope,nope,D,own", [(4, 96, 64, 32, 32, 128, True), (3, 10, 12, 4, 8, 64, True),
-                                                      (5, 7, 200, 56, 6, 256, True), (2, 6, 12, 4, 8, 64, False)])
-def test_latent_prep(H, qlr, lat, rope, nope, D, own, dt):
+@pytest.mark.parametrize("H,qlr,lat,rope,nope,D,off,own,vals", [
+    (4, 96, 64, 32, 32, 128, 64, True, True), (3, 10, 12, 4, 8, 64, 12, True, True),
+    (5, 7, 200, 56, 6, 256, 200, True, True), (2, 6, 12, 4, 8, 64, 12, False, True),
+    (4, 96, 64, 32, 32, 96, 64, True, False), (3, 10, 12, 4, 8, 96, 64, True, False),    # key rows only
+    (5, 7, 200, 56, 6, 320, 256, True, False), (2, 6, 100, 8, 8, 160, 128, False, False)])
+def test_latent_prep(H, qlr, lat, rope, nope, D, off, own, vals, dt):
     torch.manual_seed(4)
     T, P = 11, 16
     a = torch.randn(T, qlr + (lat + rope if own else 0)).to(dt)
@@ -129,12 +132,45 @@ def test_latent_prep(H, qlr, lat, rope, nope, D, own, dt):
     slots[3] = -1                                        # a padding row lands in the scratch page
     q = torch.randn(T, H, nope + rope).to(dt)
     kc, vc, qf = torch.zeros(5, 1, P, D, dtype=dt), torch.zeros(5, 1, D, P, dtype=dt), torch.full((T, H, D), 7.0, dtype=dt)
-    ref.latent_prep(a, qlr, lat, rope, w, 1e-6, pos, cs, slots, kc if own else None, vc if own else None, q, nope, qf)
+    ref.latent_prep(a, qlr, lat, rope, w, 1e-6, pos, cs, slots, kc if own else None, vc if own and vals else None, q,
+                    nope, qf, off)
     kc2, vc2, qf2 = torch.zeros_like(kc).to(DEV), torch.zeros_like(vc).to(DEV), torch.full((T, H, D), 7.0, dtype=dt).to(DEV)
     ops.latent_prep(a.to(DEV), qlr, lat, rope, w.to(DEV), 1e-6, pos.to(DEV), cs.to(DEV), slots.to(DEV),
-                    kc2 if own else None, vc2 if own else None, q.to(DEV), nope, qf2)
+                    kc2 if own else None, vc2 if own and vals else None, q.to(DEV), nope, qf2, rope_off=off)
     assert _close(kc2, kc, _tol(dt)) and _close(vc2, vc, _tol(dt)) and _close(qf2[:, :, lat:], qf[:, :, lat:], _tol(dt))
     assert torch.equal(qf2[:, :, :lat].cpu(), qf[:, :, :lat])          # the latent columns are the caller's
+    if own:
+        assert kc[:, :, :, lat:off].abs().sum() == 0 and kc[:, :, :, :lat].abs().sum() > 0      # the gap stays zero
+
+
+@pytest.mark.parametrize("shape", list(ops.LATENT_SHAPES))
+@pytest.mark.parametrize("H", [4, 16, 19])
+def test_latent_attn_kernel(shape, H):
+    """The MFMA latent kernel (key rows that carry their values, sinks) against the reference: prompt
+    chunks whose rows see different key counts, decode rows over long and short contexts (split-K
+    partials and their merge), partial pages, scattered block tables."""
+    DK, DV = shape
+    torch.manual_seed(DK + H)
+    P, n_pages = 16, 200
+    cache = (torch.randn(n_pages, P, DK, device=DEV) * 0.5).to(BF)
+    sinks = torch.randn(H, device=DEV)
+    kv_lens, q_lens = [3, 40, 1300, 97, 1], [3, 9, 20, 1, 1]
+    bt = torch.stack([torch.randperm(n_pages - 1, device=DEV)[:84] + 1 for _ in kv_lens]).to(torch.int32)
+    tok_row = torch.tensor([i for i, n in enumerate(q_lens) for _ in range(n)], dtype=torch.int32, device=DEV)
+    tok_len = torch.tensor([kv - n + j + 1 for kv, n in zip(kv_lens, q_lens) for j in range(n)], dtype=torch.int32,
+                           device=DEV)
+    q = (torch.randn(int(tok_row.numel()), H, DK, device=DEV) * 0.5).to(BF)
+    for sk in (sinks, None):
+        got = ops.latent_attn(q, cache, bt, tok_row, tok_len, 0.15, DV, sinks=sk)
+        want = ref.mla_attn(q.cpu(), cache.cpu(), bt.cpu(), tok_row.cpu(), tok_len.cpu(), 0.15, DV,
+                            None if sk is None else sk.cpu())
+        assert _close(got, want, 2e-2)
+    qd = (torch.randn(5, H, DK, device=DEV) * 0.5).to(BF)                 # decode: one row per sequence
+    rows = torch.arange(5, dtype=torch.int32, device=DEV)
+    kl = torch.tensor(kv_lens, dtype=torch.int32, device=DEV)
+    got = ops.latent_attn(qd, cache, bt, rows, kl, 0.15, DV, sinks=sinks)
+    want = ref.mla_attn(qd.cpu(), cache.cpu(), bt.cpu(), rows.cpu(), kl.cpu(), 0.15, DV, sinks.cpu())
+    assert _close(got, want, 2e-2)
 
 
 @pytest.mark.parametrize("Hq,D", [(4, 128), (6, 64), (16, 256), (5, 128)])
