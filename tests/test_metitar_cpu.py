@@ -48,6 +48,23 @@ def test_latent_attention_alone(kw):
         assert _rel(mc.run_chunks(blk, h, cuts, kv), want) < 1e-4, cuts
 
 
+@pytest.mark.parametrize("kw", [dict(), dict(heads=5, dim=4, rot_dim=2, vdim=9, kv_rank=70, q_rank=5, scale=0.5),
+                                dict(heads=18, dim=4, rot_dim=4, vdim=2, kv_rank=6, q_rank=4)])
+def test_latent_attention_key_rows_layout(kw):
+    """16-bit models keep one row per token that carries its own values (padded to a latent kernel
+    shape): the same mixer on that layout, through the reference of the latent kernel."""
+    L = mo.attention_layer(**kw)
+    _, wt = _one_layer(L)
+    w, m = mo.sub(wt, "l0.mix."), L["mixer"]
+    h = torch.randn(45, 24, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    want = mo.latent_attention(h.to(F64), _w64(w), m, 1e-5)
+    for cuts in ([45], [40] + [1] * 5, [2, 3, 17, 16, 1, 6]):
+        blk, kv = mc.attention_block(m, 24, DEV, torch.bfloat16)
+        blk.load(w)
+        assert blk.latent_cache and (blk.D, blk.DV) in ops.LATENT_SHAPES
+        assert _rel(mc.run_chunks(blk, h, cuts, kv), want) < 0.05, cuts
+
+
 def test_sink_matters():
     """Leaving the sink out of the denominator changes the first rows most (few keys beside it)."""
     L = mo.attention_layer()
