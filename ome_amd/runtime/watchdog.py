@@ -29,6 +29,7 @@ import os
 import sys
 import threading
 import time
+import weakref
 from typing import Callable
 
 log = logging.getLogger("ome_amd.watchdog")
@@ -103,6 +104,16 @@ def maybe_inject(rank: int, step: int, fault: dict | None) -> bool:
     return n > 0
 
 
+_live: "weakref.WeakSet[Watchdog]" = weakref.WeakSet()   # every watchdog whose monitor thread may still run
+
+
+def stop_all() -> None:
+    """Stop every live monitor thread (a process that drops its engines without ``shutdown``, e.g.
+    a test session, would otherwise keep them polling the process-wide communicator registry)."""
+    for wd in list(_live):
+        wd.stop()
+
+
 class Watchdog:
     """Phase tracker + monitor thread.  ``enter(phase)`` at each phase boundary, ``idle()`` when the
     loop has nothing in flight; ``on_fire(code, reason)`` defaults to logging + ``os._exit(code)``."""
@@ -117,6 +128,7 @@ class Watchdog:
         self.t_phase = time.monotonic()
         self.fired: tuple[int, str] | None = None
         self._stop = threading.Event()
+        _live.add(self)
         self._t = threading.Thread(target=self._run, name="ome-watchdog", daemon=True)
         self._t.start()
 
@@ -161,4 +173,4 @@ class Watchdog:
 
 
 __all__ = ["CommError", "EXIT_COLLECTIVE", "EXIT_STUCK", "Watchdog", "check_comms", "comm_errors", "maybe_inject",
-           "parse_fault", "register_comm", "unregister_all"]
+           "parse_fault", "register_comm", "stop_all", "unregister_all"]

@@ -29,3 +29,14 @@ def pytest_collection_modifyitems(config, items):
     for it in items:
         if "gpu" in it.keywords:
             it.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def _stop_leftover_watchdogs():
+    """Engines that tests drop without ``shutdown`` leave their watchdog threads polling the
+    process-wide communicator registry; a later test that records a collective error there on
+    purpose would be ended by one of them (exit 75).  Stop them when the test that made them ends."""
+    yield
+    from ome_amd.runtime import watchdog
+
+    watchdog.stop_all()
