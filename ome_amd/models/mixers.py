@@ -295,6 +295,9 @@ class LatentAttention(_Block):
         else:
             self.D = latent_row_width(kv_rank, rot_dim)
             self.DV = kv_rank
+            if dtype != torch.float32 and self.D > 256:
+                raise ValueError(f"latent attention: a {kv_rank} + {rot_dim}-wide row fits neither the latent kernel "
+                                 "(latent <= 512, rotary <= 64) nor the 256-wide attention tile")
         self.cos_sin = yarn_rope_table(rot_base, rot_dim, max_positions, rot_scaling, self.device)
         self.w_in = self.qn = self.w_uq = self.kvn = self.w_uk = self.w_uv = self.sink = self.w_o = None
 
@@ -350,6 +353,7 @@ class LatentAttention(_Block):
 
 
 _ARANGE: dict = {}
+_ARANGE_KEEP: list = []
 _LATENT_WS: dict = {}
 
 
@@ -361,6 +365,7 @@ def latent_rows(meta: AttnMeta, T: int) -> list:
     ar = _ARANGE.get(dev)
     if ar is None or ar.numel() < T:
         ar = _ARANGE[dev] = torch.arange(max(T, 4096), dtype=torch.int32, device=dev)
+        _ARANGE_KEEP.append(ar)    # (captured decode graphs keep reading the one they were recorded with)
     if meta.is_decode:
         return [(0, T, meta.block_tables, ar[:T], meta.seq_lens)]
     kv_lens = (meta.positions + 1).to(torch.int32)
